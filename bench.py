@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the binary-convolution hot path on one MI355X.
+
+Headline workload (BASELINE.json config 3 at batch 64): one "step" is one pass
+of the direct 3x3 binary convolution over the seven ResNet-18 stage shapes
+(56/64, 28/128, 14/256, 7/512 at stride 1 and the three stride-2 channel
+doubling layers), packed activations and weights already resident in HBM,
+fp32 mismatch counts written back.  value = binary ops per second,
+binops = 2*N*OH*OW*Cout*9*Cin.
+
+The same JSON line also carries, under "workloads", the other BASELINE
+configurations (single 56x56x64 layer at batch 1, standalone bitpack and bgemm,
+the whole BinConv layer from fp32 input), the VALU-popcount roofline of the
+dominant kernel and the CPU baseline (the oracle's restatement of the
+reference's generic x86 path, timed on this host).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+STAGE_SHAPES = [  # (H=W, Cin, Cout, stride)
+    (56, 64, 64, 1), (28, 128, 128, 1), (14, 256, 256, 1), (7, 512, 512, 1),
+    (56, 64, 128, 2), (28, 128, 256, 2), (14, 256, 512, 2),
+]
+BATCH = 64
+
+
+def out_dim(size, pad, k, stride):
+    return (size + 2 * pad - k) // stride + 1
+
+
+def binops(n, hw, cin, cout, stride):
+    o = out_dim(hw, 1, 3, stride)
+    return 2 * n * o * o * cout * 9 * cin
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path has no exchange between images, run it with --gpus 1 "
+                 "(a multi-GPU figure is N independent copies of this run)")
+
+    import numpy as np
+    import torch
+
+    import dabnn_amd as dab
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    cus, khz = dab.capi.device_info()
+    peak_binops = cus * 64 * (khz * 1e3) * 32  # one v_xor_b32 + one v_bcnt_u32_b32 per 32 bits per lane
+
+    g = torch.Generator(device="cpu").manual_seed(1234)
+
+    def rand_words(*shape):
+        return torch.randint(-2**63, 2**63 - 1, shape, dtype=torch.int64, generator=g).cuda()
+
+    def timed(fn, reps):
+        """Average duration of fn() over reps back-to-back launches, HIP events on the launch stream."""
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    # ------------------------------------------------------------ headline: 7 stage shapes at batch 64
+    layers = []
+    for (hw, cin, cout, stride) in STAGE_SHAPES:
+        x = rand_words(BATCH, hw, hw, cin // 64)
+        w = rand_words(cout, 9 * cin // 64)
+        layers.append((x, w, stride, binops(BATCH, hw, cin, cout, stride)))
+    step_binops = sum(l[3] for l in layers)
+
+    def step():
+        for (x, w, stride, _) in layers:
+            dab.bconv_3x3(x, w, stride, 1)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = step_binops * args.steps / wall
+
+    # per-shape kernel durations (the roofline figure is launch-level)
+    per_shape = []
+    dur_sum = 0.0
+    for (hw, cin, cout, stride), (x, w, s, ops) in zip(STAGE_SHAPES, layers):
+        d = timed(lambda: dab.bconv_3x3(x, w, s, 1), max(20, args.steps))
+        dur_sum += d
+        per_shape.append({"shape": "%dx%d %d->%d s%d b%d" % (hw, hw, cin, cout, stride, BATCH), "us": round(d * 1e6, 2),
+                          "Tbinop/s": round(ops / d / 1e12, 1), "frac": round(ops / d / peak_binops, 3)})
+    achieved = step_binops / dur_sum
+
+    workloads = {"config3_b64_per_shape": per_shape,
+                 "config3_b64_events_ms_per_step": round(e0.elapsed_time(e1) / args.steps, 4)}
+
+    # ------------------------------------------------------------ config 3 at batch 1 and config 1
+    b1 = []
+    for (hw, cin, cout, stride) in STAGE_SHAPES:
+        x, w = rand_words(1, hw, hw, cin // 64), rand_words(cout, 9 * cin // 64)
+        d = timed(lambda: dab.bconv_3x3(x, w, stride, 1), 50)
+        b1.append({"shape": "%dx%d %d->%d s%d b1" % (hw, hw, cin, cout, stride), "us": round(d * 1e6, 2),
+                   "Gbinop/s": round(binops(1, hw, cin, cout, stride) / d / 1e9, 1)})
+    workloads["config3_b1_per_shape"] = b1
+    xf = torch.randn((1, 56, 56, 64), generator=g).cuda()
+    layer = dab.BinConv(rand_words(64, 9), 3, 3, 1, 1, 1, 1)
+    d = timed(lambda: layer(xf), 50)
+    workloads["config1_binconv_fp32_in_b1"] = {"us": round(d * 1e6, 2),
+                                               "Gbinop/s": round(binops(1, 56, 64, 64, 1) / d / 1e9, 1)}
+
+    # ------------------------------------------------------------ config 2: standalone bitpack and bgemm
+    xp = torch.randn((1, 56, 56, 512), generator=g).cuda()
+    d = timed(lambda: dab.pack_mat(xp), 200)
+    pack_bytes = xp.numel() * 4 + xp.numel() // 8
+    workloads["config2_bitpack_1x512x56x56"] = {"us": round(d * 1e6, 2), "GB/s": round(pack_bytes / d / 1e9, 1),
+                                                "frac_hbm_8TBs": round(pack_bytes / d / 8e12, 3)}
+    xpb = torch.randn((64, 56, 56, 512), generator=g).cuda()
+    d = timed(lambda: dab.pack_mat(xpb), 20)
+    workloads["bitpack_64x56x56x512"] = {"us": round(d * 1e6, 2), "GB/s": round(64 * pack_bytes / d / 1e9, 1),
+                                         "frac_hbm_8TBs": round(64 * pack_bytes / d / 8e12, 3)}
+    del xpb
+    m, n, k = 512, 3136, 72
+    a, b = rand_words(k, m), rand_words(n, k)
+    c = torch.zeros((n, m), dtype=torch.float32, device="cuda")
+    d = timed(lambda: dab.bgemm(m, n, k, a, m, b, k, c, m), 50)
+    gemm_ops = 2 * m * n * k * 64
+    workloads["config2_bgemm_m512_k72_n3136"] = {"us": round(d * 1e6, 2), "Tbinop/s": round(gemm_ops / d / 1e12, 1),
+                                                 "frac": round(gemm_ops / d / peak_binops, 3)}
+    xi = torch.randn((64, 28, 28, 128), generator=g).cuda()
+    d = timed(lambda: dab.fused_binarize_im2col(xi, 3, 3, 1, 1, 1, 1), 50)
+    im_bytes = xi.numel() * 4 + 64 * 28 * 28 * 18 * 8
+    workloads["fused_binarize_im2col_64x28x28x128"] = {"us": round(d * 1e6, 2), "GB/s": round(im_bytes / d / 1e9, 1),
+                                                       "frac_hbm_8TBs": round(im_bytes / d / 8e12, 3)}
+
+    # ------------------------------------------------------------ whole BinConv layer (fp32 in) at batch 64
+    full = []
+    for (hw, cin, cout, stride) in STAGE_SHAPES:
+        xf = torch.randn((BATCH, hw, hw, cin), generator=g).cuda()
+        layer = dab.BinConv(rand_words(cout, 9 * cin // 64), 3, 3, 1, 1, stride, stride)
+        d = timed(lambda: layer(xf), 20)
+        ops = binops(BATCH, hw, cin, cout, stride)
+        full.append({"shape": "%dx%d %d->%d s%d b%d" % (hw, hw, cin, cout, stride, BATCH), "us": round(d * 1e6, 2),
+                     "Tbinop/s": round(ops / d / 1e12, 1)})
+    workloads["binconv_layer_fp32_in_b64"] = full
+
+    # ------------------------------------------------------------ CPU baseline (rank 0, bounded sample)
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle as orc
+        r = np.random.default_rng(7)
+        cases = []
+        for (hw, cin, cout, stride) in STAGE_SHAPES:
+            cases.append((r.standard_normal((hw, hw, cin)).astype(np.float32),
+                          orc.pack_weight(r.standard_normal((cout, 3, 3, cin)).astype(np.float32)), stride,
+                          binops(1, hw, cin, cout, stride)))
+        done_ops, t_cpu, passes = 0, 0.0, 0
+        while t_cpu < args.cpu_seconds or passes == 0:
+            t1 = time.perf_counter()
+            for (x, w, s, ops) in cases:
+                orc.binconv_forward(x, w, 3, 3, 1, 1, s, s)
+                done_ops += ops
+            t_cpu += time.perf_counter() - t1
+            passes += 1
+        cpu = {"value": done_ops / t_cpu, "unit": "binop/s", "cores": 1, "kind": "port",
+               "sample": "%d passes of the 7 stage shapes at batch 1 through the reference's x86 dispatch "
+                         "(pack_mat + baseline_bconv for 64 channels, fused_binarize_im2col + bgemm_naive "
+                         "otherwise), fp32 input, %.1f s" % (passes, t_cpu)}
+
+    line = {
+        "metric": "bconv binary-op/s",
+        "value": value,
+        "unit": "binop/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "BASELINE config 3: binary 3x3 conv over the 7 ResNet-18 stage shapes, batch 64, "
+                               "stride 1/2, pad 1, packed uint64 activations in, fp32 counts out",
+                   "batch": BATCH, "binops_per_step": step_binops, "device": torch.cuda.get_device_name(0),
+                   "cus": cus, "clock_mhz": khz / 1e3},
+        "roofline": {"bound": "valu_popcount", "achieved": achieved / 1e12, "peak": peak_binops / 1e12,
+                     "unit": "Tbinop/s", "frac": achieved / peak_binops, "traffic": None,
+                     "kernel": "bconv3x3_kernel", "note": "peak = CUs*64 lanes*clock*32 binop (one v_xor_b32 + one "
+                     "v_bcnt_u32_b32 per 32 bits); achieved = sum of binops / sum of per-shape average launch durations"},
+        "cpu_baseline": cpu,
+        "workloads": workloads,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,25 @@
+"""MI355X (gfx950) backend for the binary-convolution path of dabnn.
+
+The compute lives in ``lib/libdabnn_hip.so`` (hand-written HIP kernels behind
+the C ABI declared in ``include/dabnn_hip.h``).  This package is the thin
+Python plumbing over it: it hands device pointers of torch tensors to the C
+ABI and mirrors the reference's function names.  There is no CPU fallback:
+importing :mod:`dabnn_amd.capi` raises when the library has not been built.
+"""
+from . import capi  # noqa: F401
+from .ops import (  # noqa: F401
+    BinConv,
+    add_inplace,
+    affine_inplace,
+    ave_pool,
+    bconv_3x3,
+    bgemm,
+    bitpack_nchw,
+    col_row_words,
+    fconv,
+    fused_binarize_im2col,
+    max_pool,
+    pack_mat,
+    pad,
+    weight_transpose,
+)

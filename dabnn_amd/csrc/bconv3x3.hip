@@ -1,0 +1,157 @@
+// Direct 3x3 binary convolution for 64/128/256/512 input channels.
+//
+// Replaces the reference's pack -> pad -> bconv_3x3 chain
+// (dabnn/layers/BinConv.cpp:145-150, dabnn/bconv.h:855-931) on packed input;
+// results equal baseline_bconv (common/baseline.h:77-116) bit for bit.
+//
+// Data layout: x [N][H][W][CW] uint64 (CW = cin/64), weights in the reference's
+// own order [cout][3][3][CW] (no repacking), out [N][OH][OW][cout] fp32.
+// A lane owns one output pixel and keeps its 9*CW input words (18*CW VGPRs)
+// resident; out-of-image taps are fetched through a buffer descriptor with an
+// out-of-range offset, which the hardware answers with zero -- the zero word
+// that stands for 64 values of -1 (dabnn/pad.h:12).
+#include "xnor_core.h"
+
+namespace dab {
+
+struct BconvArgs {
+    const uint64_t *x;
+    const uint64_t *w;
+    float *out;
+    int total;     // N*OH*OW output pixels
+    int H, W, OH, OW;
+    int cout;
+    int stride, pad;
+    int n_groups;  // cout / 8
+    int n_units;   // tiles * n_groups
+    int n_waves;
+    uint32_t x_bytes;
+    FastDiv div_ow, div_oh;
+};
+
+constexpr int kWavesPerBlock = 4;
+
+template <int CW>
+__global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const BconvArgs p) {
+    constexpr int K32 = 18 * CW;
+    __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    unsigned char *stage = stage_all + wib * kStageBytes;
+    const int wv = blockIdx.x * kWavesPerBlock + wib;
+
+    int u0, u1;
+    unit_range(wv, p.n_waves, p.n_units, u0, u1);
+    if (u0 >= u1) return;
+
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
+    int tile = u0 / p.n_groups;
+    int cg = u0 - tile * p.n_groups;
+    int g_lo = cg & 3;
+    bool need_load = true;
+    uint32_t a[K32];
+
+    for (int u = u0; u < u1; ++u) {
+        if (need_load) {
+            need_load = false;
+            int pix = tile * 64 + lane;
+            pix = pix < p.total ? pix : p.total - 1;
+            const uint32_t t = p.div_ow.div(pix);
+            const int ox = pix - t * p.OW;
+            const uint32_t n = p.div_oh.div(t);
+            const int oy = t - n * p.OH;
+            const int y0 = oy * p.stride - p.pad, x0 = ox * p.stride - p.pad;
+            const int base = ((n * p.H + y0) * p.W + x0) * (CW * 8);  // byte offset of tap (0,0); may be negative
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh) {
+                const bool row_ok = (unsigned)(y0 + kh) < (unsigned)p.H;
+#pragma unroll
+                for (int kw = 0; kw < 3; ++kw) {
+                    const bool ok = row_ok && (unsigned)(x0 + kw) < (unsigned)p.W;
+                    // an offset beyond the descriptor's range reads as zero
+                    const int off = ok ? base + (kh * p.W + kw) * (CW * 8) : (int)0x80000000;
+                    uint32_t *dst = a + (kh * 3 + kw) * CW * 2;
+                    if constexpr (CW == 1) {
+                        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+                        dst[0] = v.x, dst[1] = v.y;
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < CW / 2; ++c) {
+                            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, c * 16, 0);
+                            dst[4 * c] = v.x, dst[4 * c + 1] = v.y, dst[4 * c + 2] = v.z, dst[4 * c + 3] = v.w;
+                        }
+                    }
+                }
+            }
+        }
+
+        uint32_t acc[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc[q] = kAccInit;
+        unit_rowmajor<K32>(p.w + (size_t)cg * 8 * (9 * CW), a, acc);
+        stage_put(stage, lane, cg & 3, acc);
+
+        const bool last_in_tile = cg == p.n_groups - 1;
+        if ((cg & 3) == 3 || last_in_tile || u == u1 - 1) {
+            stage_flush<false>(stage, lane, p.out, p.cout, tile, p.total, (cg & ~3) * 8, g_lo, cg & 3);
+            g_lo = 0;
+        }
+        if (last_in_tile) {
+            cg = 0;
+            ++tile;
+            need_load = true;
+        } else {
+            ++cg;
+        }
+    }
+}
+
+template <int CW>
+static int launch_bconv3x3(const BconvArgs &args, hipStream_t stream) {
+    hipLaunchKernelGGL(bconv3x3_kernel<CW>, dim3(args.n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream,
+                       args);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+}  // namespace dab
+
+extern "C" int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
+                            int pad, float *out, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && wgt && out, "dab_bconv3x3: null pointer");
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0, "dab_bconv3x3: non-positive dimension");
+    DAB_REQUIRE(stride > 0 && pad >= 0, "dab_bconv3x3: stride %d pad %d", stride, pad);
+    DAB_REQUIRE(cin % 64 == 0, "dab_bconv3x3: cin %d is not a multiple of 64", cin);
+    DAB_REQUIRE(h + 2 * pad >= 3 && w + 2 * pad >= 3, "dab_bconv3x3: input smaller than the kernel");
+    if (!(cin == 64 || cin == 128 || cin == 256 || cin == 512) || cout % 8 != 0)
+        return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: cin %d / cout %d not covered by the direct kernel", cin, cout);
+    DAB_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wgt) & 7) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & 15) == 0,
+                "dab_bconv3x3: buffers must be 16-byte aligned");
+
+    BconvArgs a;
+    a.x = x, a.w = wgt, a.out = out;
+    a.H = h, a.W = w;
+    a.OH = out_dim(h, pad, 3, 1, stride), a.OW = out_dim(w, pad, 3, 1, stride);
+    const long long total = (long long)n * a.OH * a.OW;
+    const long long x_bytes = (long long)n * h * w * (cin / 64) * 8;
+    if (total >= (1ll << 31) - 64 || x_bytes >= (1ll << 31) || total * cout >= (1ll << 40))
+        return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: tensor too large for 32-bit pixel indexing");
+    a.total = (int)total;
+    a.cout = cout, a.stride = stride, a.pad = pad;
+    a.n_groups = cout / 8;
+    const long long units = ((total + 63) / 64) * a.n_groups;
+    if (units >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
+    a.n_units = (int)units;
+    a.n_waves = pick_wave_count(a.n_units, 4, kWavesPerBlock);
+    a.x_bytes = (uint32_t)x_bytes;
+    a.div_ow = FastDiv((uint32_t)a.OW), a.div_oh = FastDiv((uint32_t)a.OH);
+    hipStream_t s = as_stream(stream);
+    switch (cin) {
+        case 64: return launch_bconv3x3<1>(a, s);
+        case 128: return launch_bconv3x3<2>(a, s);
+        case 256: return launch_bconv3x3<4>(a, s);
+        default: return launch_bconv3x3<8>(a, s);
+    }
+}

@@ -1,0 +1,147 @@
+// Sign bit-packing and the small data-movement helpers around it.
+//
+// Packing rule (common/common_bitpack.h:26,110-174): bit j of word i is 1 iff
+// x[64*i + j] > 0 (so +0, -0, NaN and negatives give 0).  On a 64-lane wave
+// that is exactly one v_cmp_gt_f32: the lane mask it produces IS the word.
+// A wave therefore reads 64 consecutive floats per instruction (256 coalesced
+// bytes), keeps the 64 masks of a 16 KiB chunk in lane i of a register pair
+// and writes them with one coalesced 512-byte store.  HBM-bound: 4 bytes read
+// and 1/16 byte written per element.
+#include "common.h"
+
+namespace dab {
+
+constexpr int kPackWavesPerBlock = 4;
+
+__global__ __launch_bounds__(64 * kPackWavesPerBlock) void bitpack_nhwc_kernel(const float *__restrict__ x,
+                                                                              uint64_t *__restrict__ out,
+                                                                              long long n_words) {
+    const int lane = threadIdx.x & 63;
+    const long long wave = (long long)blockIdx.x * kPackWavesPerBlock + (threadIdx.x >> 6);
+    const long long n_chunks = (n_words + 63) / 64;
+    const long long stride = (long long)gridDim.x * kPackWavesPerBlock;
+    for (long long chunk = wave; chunk < n_chunks; chunk += stride) {
+        const long long w0 = chunk * 64;
+        const float *src = x + w0 * 64 + lane;
+        uint64_t mine = 0;
+        if (w0 + 64 <= n_words) {
+#pragma unroll 16
+            for (int i = 0; i < 64; ++i) {
+                const uint64_t word = __ballot(src[(long long)i * 64] > 0.0f);
+                mine = (lane == i) ? word : mine;
+            }
+            out[w0 + lane] = mine;
+        } else {
+            const int rem = (int)(n_words - w0);
+            for (int i = 0; i < rem; ++i) {
+                const uint64_t word = __ballot(src[(long long)i * 64] > 0.0f);
+                mine = (lane == i) ? word : mine;
+            }
+            if (lane < rem) out[w0 + lane] = mine;
+        }
+    }
+}
+
+// NCHW input: a lane owns one pixel and walks the 64 channels of a word, so
+// the loads of a wave are 64 consecutive floats of one channel plane.
+__global__ __launch_bounds__(256) void bitpack_nchw_kernel(const float *__restrict__ x, uint64_t *__restrict__ out,
+                                                           int n, int cw, long long hw) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;  // over n * cw * hw, pixel fastest
+    const long long total = (long long)n * cw * hw;
+    if (idx >= total) return;
+    const long long pix = idx % hw;
+    const long long t = idx / hw;
+    const int k = (int)(t % cw);
+    const long long img = t / cw;
+    const float *src = x + ((img * cw + k) * 64) * hw + pix;
+    uint32_t lo = 0, hi = 0;
+#pragma unroll 8
+    for (int j = 0; j < 32; ++j) lo |= (src[(long long)j * hw] > 0.0f ? 1u : 0u) << j;
+#pragma unroll 8
+    for (int j = 0; j < 32; ++j) hi |= (src[(long long)(j + 32) * hw] > 0.0f ? 1u : 0u) << j;
+    out[(img * hw + pix) * cw + k] = ((uint64_t)hi << 32) | lo;
+}
+
+__global__ __launch_bounds__(256) void pad_bit_kernel(const uint64_t *__restrict__ x, uint64_t *__restrict__ out, int n,
+                                                      int h, int w, int cw, int pad_h, int pad_w) {
+    const int oh = h + 2 * pad_h, ow = w + 2 * pad_w;
+    const long long total = (long long)n * oh * ow * cw;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int c = (int)(idx % cw);
+    long long t = idx / cw;
+    const int xo = (int)(t % ow);
+    t /= ow;
+    const int yo = (int)(t % oh);
+    const long long img = t / oh;
+    const int yi = yo - pad_h, xi = xo - pad_w;
+    uint64_t v = 0;
+    if (yi >= 0 && yi < h && xi >= 0 && xi < w) v = x[((img * h + yi) * w + xi) * cw + c];
+    out[idx] = v;
+}
+
+__global__ __launch_bounds__(256) void weight_transpose_kernel(const uint64_t *__restrict__ w, uint64_t *__restrict__ wt,
+                                                               int m, int k) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;  // over k*m, m fastest (coalesced writes)
+    if (idx >= (long long)m * k) return;
+    const int j = (int)(idx % m);
+    const int i = (int)(idx / m);
+    wt[idx] = w[(size_t)j * k + i];
+}
+
+static unsigned blocks_for(long long total, int per_block) {
+    long long b = (total + per_block - 1) / per_block;
+    return (unsigned)(b < 1 ? 1 : b);
+}
+
+}  // namespace dab
+
+extern "C" int dab_bitpack_nhwc(const float *x, uint64_t *out, int64_t n_pix, int c, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && out, "dab_bitpack_nhwc: null pointer");
+    DAB_REQUIRE(n_pix > 0 && c > 0, "dab_bitpack_nhwc: n_pix %lld c %d", (long long)n_pix, c);
+    DAB_REQUIRE(c % 64 == 0, "dab_bitpack_nhwc: c %d is not a multiple of 64", c);
+    const long long n_words = (long long)n_pix * (c / 64);
+    const long long chunks = (n_words + 63) / 64;
+    long long blocks = (chunks + kPackWavesPerBlock - 1) / kPackWavesPerBlock;
+    const long long cap = (long long)simd_count() * 8;  // grid-stride beyond 8 waves per SIMD
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(bitpack_nhwc_kernel, dim3((unsigned)blocks), dim3(64 * kPackWavesPerBlock), 0, as_stream(stream), x,
+                       out, n_words);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_bitpack_nchw(const float *x, uint64_t *out, int n, int c, int h, int w, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && out, "dab_bitpack_nchw: null pointer");
+    DAB_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0, "dab_bitpack_nchw: non-positive dimension");
+    DAB_REQUIRE(c % 64 == 0, "dab_bitpack_nchw: c %d is not a multiple of 64", c);
+    const long long total = (long long)n * (c / 64) * h * w;
+    hipLaunchKernelGGL(bitpack_nchw_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, as_stream(stream), x, out, n,
+                       c / 64, (long long)h * w);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_pad_bit(const uint64_t *x, int n, int h, int w, int cw, int pad_h, int pad_w, uint64_t *out,
+                           dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && out, "dab_pad_bit: null pointer");
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && cw > 0 && pad_h >= 0 && pad_w >= 0, "dab_pad_bit: bad dimension");
+    const long long total = (long long)n * (h + 2 * pad_h) * (w + 2 * pad_w) * cw;
+    hipLaunchKernelGGL(pad_bit_kernel, dim3(blocks_for(total, 256)), dim3(256), 0, as_stream(stream), x, out, n, h, w, cw,
+                       pad_h, pad_w);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_weight_transpose(const uint64_t *w, int m, int k, uint64_t *wt, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(w && wt, "dab_weight_transpose: null pointer");
+    DAB_REQUIRE(m > 0 && k > 0, "dab_weight_transpose: m %d k %d", m, k);
+    hipLaunchKernelGGL(weight_transpose_kernel, dim3(blocks_for((long long)m * k, 256)), dim3(256), 0, as_stream(stream),
+                       w, wt, m, k);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}

@@ -1,0 +1,122 @@
+// fused_binarize_im2col (dabnn/fused_binarize_im2col.h:6-68) on the GPU.
+//
+// Output: one row per output pixel, each row = the kh*kw*c gathered floats
+// (zeros where a tap falls outside the image) zero-extended to a multiple of
+// 128 and sign-packed; row_words = ceil(kh*kw*c/128)*2 words.
+//
+// A wave produces one output word per compare: lane l looks at element
+// 64*wi + l of the row and the lane mask of (value > 0) is the word.  When c
+// is a multiple of 64 a word never straddles two taps, so tap position and
+// bounds test are wave-uniform (scalar) and the 64 lanes read 256 contiguous
+// bytes.  The general path resolves tap and channel per lane.
+// HBM-bound on paper (each input float is needed kh*kw times but comes from
+// L2 after the first touch): 4 bytes per input element read, 8 bytes per
+// output word written.
+#include "common.h"
+
+namespace dab {
+
+struct Im2colArgs {
+    const float *x;
+    uint64_t *col;
+    int n, h, w, c;
+    int kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w;
+    int oh, ow;
+    int row_words;
+    int len;  // kh*kw*c
+    long long n_words;
+    FastDiv div_row_words, div_ow, div_oh, div_c, div_kw, div_cw;
+};
+
+constexpr int kIm2colWavesPerBlock = 4;
+
+template <bool ALIGNED64>
+__global__ __launch_bounds__(64 * kIm2colWavesPerBlock) void fused_binarize_im2col_kernel(const Im2colArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long wave = (long long)blockIdx.x * kIm2colWavesPerBlock + wib;
+    const long long n_chunks = (p.n_words + 63) / 64;
+    const long long stride = (long long)gridDim.x * kIm2colWavesPerBlock;
+    for (long long chunk = wave; chunk < n_chunks; chunk += stride) {
+        const long long g0 = chunk * 64;
+        const int count = (int)(p.n_words - g0 < 64 ? p.n_words - g0 : 64);
+        uint64_t mine = 0;
+        for (int i = 0; i < count; ++i) {
+            const uint32_t g = (uint32_t)(g0 + i);  // global word index (n_words < 2^31 checked on the host)
+            const uint32_t row = p.div_row_words.div(g);
+            const int wi = g - row * p.row_words;
+            const uint32_t t = p.div_ow.div(row);
+            const int ox = row - t * p.ow;
+            const uint32_t img = p.div_oh.div(t);
+            const int oy = t - img * p.oh;
+            float v = 0.0f;
+            if constexpr (ALIGNED64) {
+                const int cw = p.c >> 6;
+                const uint32_t tap = p.div_cw.div((uint32_t)wi);  // >= kh*kw for the zero padding word
+                const int k = wi - tap * cw;
+                const uint32_t a = p.div_kw.div(tap);
+                const int b = tap - a * p.kw;
+                const int y = oy * p.stride_h - p.pad_h + (int)a * p.dil_h;
+                const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
+                if ((int)tap < p.kh * p.kw && y >= 0 && y < p.h && xx >= 0 && xx < p.w)
+                    v = p.x[(((size_t)img * p.h + y) * p.w + xx) * p.c + k * 64 + lane];
+            } else {
+                const int e = wi * 64 + lane;
+                if (e < p.len) {
+                    const uint32_t tap = p.div_c.div((uint32_t)e);
+                    const int ch = e - tap * p.c;
+                    const uint32_t a = p.div_kw.div(tap);
+                    const int b = tap - a * p.kw;
+                    const int y = oy * p.stride_h - p.pad_h + (int)a * p.dil_h;
+                    const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
+                    if (y >= 0 && y < p.h && xx >= 0 && xx < p.w) v = p.x[(((size_t)img * p.h + y) * p.w + xx) * p.c + ch];
+                }
+            }
+            const uint64_t word = __ballot(v > 0.0f);
+            mine = (lane == i) ? word : mine;
+        }
+        if (lane < count) p.col[g0 + lane] = mine;
+    }
+}
+
+}  // namespace dab
+
+extern "C" int dab_col_row_words(int kh, int kw, int c) { return (kh * kw * c + 127) / 128 * 2; }
+
+extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                                         int stride_h, int stride_w, int dil_h, int dil_w, uint64_t *col,
+                                         dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && col, "dab_fused_binarize_im2col: null pointer");
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && kh > 0 && kw > 0, "dab_fused_binarize_im2col: non-positive dimension");
+    DAB_REQUIRE(pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0,
+                "dab_fused_binarize_im2col: bad pad/stride/dilation");
+    DAB_REQUIRE((long long)kh * kw * c < 60000, "kernel_h * kernel_w * im.c must be smaller than 60000");
+    Im2colArgs a;
+    a.x = x, a.col = col;
+    a.n = n, a.h = h, a.w = w, a.c = c;
+    a.kh = kh, a.kw = kw, a.pad_h = pad_h, a.pad_w = pad_w;
+    a.stride_h = stride_h, a.stride_w = stride_w, a.dil_h = dil_h, a.dil_w = dil_w;
+    a.oh = out_dim(h, pad_h, kh, dil_h, stride_h), a.ow = out_dim(w, pad_w, kw, dil_w, stride_w);
+    DAB_REQUIRE(a.oh > 0 && a.ow > 0, "dab_fused_binarize_im2col: empty output");
+    a.len = kh * kw * c;
+    a.row_words = dab_col_row_words(kh, kw, c);
+    a.n_words = (long long)n * a.oh * a.ow * a.row_words;
+    if (a.n_words >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_fused_binarize_im2col: more than 2^31 output words");
+    a.div_row_words = FastDiv((uint32_t)a.row_words);
+    a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
+    a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv((uint32_t)kw);
+    a.div_cw = FastDiv((uint32_t)(c >= 64 ? c / 64 : 1));
+    const long long chunks = (a.n_words + 63) / 64;
+    long long blocks = (chunks + kIm2colWavesPerBlock - 1) / kIm2colWavesPerBlock;
+    const long long cap = (long long)simd_count() * 8;
+    if (blocks > cap) blocks = cap;
+    if (c % 64 == 0)
+        hipLaunchKernelGGL(fused_binarize_im2col_kernel<true>, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock), 0,
+                           as_stream(stream), a);
+    else
+        hipLaunchKernelGGL(fused_binarize_im2col_kernel<false>, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock),
+                           0, as_stream(stream), a);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}

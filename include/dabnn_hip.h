@@ -1,0 +1,162 @@
+/*
+ * C ABI of the MI355X (gfx950) backend for dabnn's binary-convolution path.
+ *
+ * Every entry point is the device-side replacement of one function of the
+ * reference (cited per declaration).  All tensor pointers are DEVICE pointers
+ * into contiguous buffers in the reference's layouts:
+ *
+ *   fp32 activations   [N][H][W][C]            (dabnn/mat.h:36, NHWC)
+ *   packed activations [N][H][W][C/64] uint64  bit j of word i = (x[64*i+j] > 0)
+ *                                              (common/common_bitpack.h:26,110-174)
+ *   packed weights     [Cout][words per filter] uint64, tap order (kh, kw, c)
+ *                                              (tools/onnx2bnn/OnnxConverter.cpp:121-156)
+ *
+ * The batch dimension N is an extension: the reference processes one image
+ * per call (dabnn/net.cpp:64-65); N images here give exactly the results of N
+ * reference calls.
+ *
+ * Calls are asynchronous on `stream` (a hipStream_t passed as void*; NULL is
+ * the default stream).  Return value: DAB_OK or a negative DAB_E* code; the
+ * functions never throw and never abort.  dab_last_error() returns a
+ * thread-local message for the last failing call.  The reference signals the
+ * same conditions with BNN_ASSERT -> std::runtime_error (common/helper.h:69-77);
+ * the C++ layer on top of this header rethrows them as that type.
+ */
+#ifndef DABNN_HIP_H
+#define DABNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define DAB_API __attribute__((visibility("default")))
+#else
+#define DAB_API
+#endif
+
+#define DAB_OK 0
+#define DAB_EINVAL (-1)      /* argument violates a reference assertion (shape, alignment, null) */
+#define DAB_EUNSUPPORTED (-2) /* valid request outside what this entry point implements */
+#define DAB_EHIP (-3)        /* a HIP runtime call failed; message holds hipGetErrorString */
+
+typedef void *dab_stream_t;
+
+/* Library / device information. */
+DAB_API const char *dab_last_error(void);
+DAB_API int dab_version(void);
+/* CU count and shader clock (kHz) of the current device; feeds the roofline figures. */
+DAB_API int dab_device_info(int *cu_count, int *clock_khz);
+
+/*
+ * pack_mat -> pack_mat_64 (dabnn/bitpack.h:254-293): sign-pack n_pix pixels of
+ * c channels (c % 64 == 0) along the channel axis.  out holds n_pix * c/64 words.
+ */
+DAB_API int dab_bitpack_nhwc(const float *x, uint64_t *out, int64_t n_pix, int c, dab_stream_t stream);
+
+/*
+ * Same output words from an NCHW tensor [n][c][h][w].  No counterpart in the
+ * reference (its tensors are NHWC only, dabnn/mat.h:36); specified as
+ * dab_bitpack_nhwc applied to the NHWC permutation of x.
+ */
+DAB_API int dab_bitpack_nchw(const float *x, uint64_t *out, int n, int c, int h, int w, dab_stream_t stream);
+
+/*
+ * pad, Bit branch (dabnn/pad.h:7-19): copy [n][h][w][cw] words into the
+ * centre of a zero-filled [n][h+2*pad_h][w+2*pad_w][cw] buffer.
+ */
+DAB_API int dab_pad_bit(const uint64_t *x, int n, int h, int w, int cw, int pad_h, int pad_w, uint64_t *out,
+                dab_stream_t stream);
+
+/*
+ * fused_binarize_im2col (dabnn/fused_binarize_im2col.h:6-68): for every
+ * output pixel gather kh*kw runs of c floats (zeros outside the image),
+ * zero-extend to a multiple of 128 floats and sign-pack.
+ * col holds n*oh*ow rows of dab_col_row_words(kh, kw, c) words.
+ * Fails with DAB_EINVAL when kh*kw*c >= 60000 (reference assertion, :14).
+ */
+DAB_API int dab_fused_binarize_im2col(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                              int stride_h, int stride_w, int dil_h, int dil_w, uint64_t *col, dab_stream_t stream);
+DAB_API int dab_col_row_words(int kh, int kw, int c);
+
+/*
+ * bgemm / bgemm_naive (dabnn/bgemm.h:46-66,587-597): column-major
+ * C(i,j) += float(popcount(A(i,h) ^ B(h,j))), A(i,h) = a[h*lda+i],
+ * B(h,j) = b[j*ldb+h], C(i,j) = c[j*ldc+i].  C is accumulated into, as in the
+ * reference (callers zero-fill it first, dabnn/layers/BinConv.cpp:153,168).
+ * Bit-exact with the reference whenever C holds integer-valued floats and
+ * every sum stays below 2^24 (always true for zero-filled C and k <= 2^18).
+ */
+DAB_API int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c, int ldc,
+              dab_stream_t stream);
+
+/*
+ * Weight transpose done by the BinConv constructor for its bgemm method
+ * (dabnn/layers/BinConv.cpp:59-76): wt[i*m + j] = w[j*k + i].
+ */
+DAB_API int dab_weight_transpose(const uint64_t *w, int m, int k, uint64_t *wt, dab_stream_t stream);
+
+/*
+ * bconv_3x3 on top of pad (dabnn/bconv.h:855-931 with dabnn/pad.h, i.e. the
+ * DIRECT_CONV arm of dabnn/layers/BinConv.cpp:145-150) == baseline_bconv
+ * (common/baseline.h:77-116) with a 3x3 kernel: x is the UNPADDED packed
+ * activation [n][h][w][cin/64]; taps outside the image read a zero word.
+ * wgt is [cout][9*cin/64] words.  out is fp32 [n][oh][ow][cout] holding the
+ * mismatch counts, oh = (h + 2*pad - 3)/stride + 1.
+ * Implemented for cin in {64, 128, 256, 512} and cout % 8 == 0; other shapes
+ * return DAB_EUNSUPPORTED (use dab_fused_binarize_im2col + dab_bgemm, as the
+ * reference's BGEMM arm does).
+ */
+DAB_API int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
+                 int pad, float *out, dab_stream_t stream);
+
+/*
+ * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
+ * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
+ * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in
+ * {64,128,256,512} takes the direct kernel (pack + bconv), anything else
+ * takes fused_binarize_im2col + bgemm on `wgt_t` (the transposed weights;
+ * may be NULL when the direct kernel applies).
+ * hwc_words = words per filter (weight.total()/weight.n).
+ * workspace must hold dab_binconv_workspace_bytes(...) bytes.
+ * method_out (optional) receives 0 = DIRECT_CONV, 1 = BGEMM.
+ */
+DAB_API size_t dab_binconv_workspace_bytes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
+                                   int stride_w);
+DAB_API int dab_binconv_forward(const float *x, int n, int h, int w, int c, const uint64_t *wgt, const uint64_t *wgt_t,
+                        int hwc_words, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int cout,
+                        float *out, void *workspace, size_t workspace_bytes, int *method_out, dab_stream_t stream);
+
+/* ------------------------------------------------------------------ float glue */
+
+/*
+ * fconv (dabnn/fconv.h:14-76): fp32 convolution, weights [cout][kh][kw][c],
+ * optional bias (NULL for none).  Agreement with the reference is to fp32
+ * rounding (1e-4 relative), the summation order differs from Eigen's.
+ */
+DAB_API int dab_fconv(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias, int kh, int kw,
+              int pad_h, int pad_w, int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *out,
+              dab_stream_t stream);
+
+/* affine_inplace (dabnn/layers/Affine.cpp:10-23): x[..., ch] = a[ch]*x[..., ch] + b[ch]. */
+DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, const float *b, dab_stream_t stream);
+
+/* add_inplace (dabnn/layers/Add.cpp:7-17): a += b over n_elem floats. */
+DAB_API int dab_add_inplace(float *a, const float *b, int64_t n_elem, dab_stream_t stream);
+
+/* ave_pool_fallback (dabnn/layers/AvePool.cpp:84-123): mean over in-bounds taps. */
+DAB_API int dab_ave_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
+                 int stride_w, float *out, dab_stream_t stream);
+
+/* max_pool_fallback (dabnn/layers/MaxPool.cpp:209-246): max over in-bounds taps from -FLT_MAX. */
+DAB_API int dab_max_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
+                 int stride_w, float *out, dab_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* DABNN_HIP_H */

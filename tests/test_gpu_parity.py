@@ -1,0 +1,299 @@
+"""GPU parity: HIP kernels (through the C ABI) vs the CPU oracle, bit-exact.
+
+Same seeded inputs go to both sides.  Sizes are chosen so the oracle finishes
+in seconds; the full BASELINE shapes at batch 64 are checked through
+size-independent properties in test_gpu_properties.py.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dab():
+    import dabnn_amd
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    return dabnn_amd
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def dev_f(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
+
+
+def dev_u(a):
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.uint64).view(np.int64)).cuda()
+
+
+def host_u(t):
+    return t.cpu().numpy().view(np.uint64)
+
+
+def special_floats(shape, seed):
+    x = rng(seed).standard_normal(shape).astype(np.float32)
+    x.flat[::7] = 0.0
+    x.flat[3::11] = -0.0
+    x.flat[5::13] = np.nan
+    x.flat[1::17] = np.float32(1e-45)
+    x.flat[2::19] = -np.float32(1e-45)
+    x.flat[4::23] = np.inf
+    x.flat[6::29] = -np.inf
+    return x
+
+
+# ---------------------------------------------------------------- bitpack
+@pytest.mark.parametrize("shape", [
+    (1, 8, 8, 128), (1, 1, 1, 64), (2, 5, 3, 192), (1, 56, 56, 64), (1, 56, 56, 512), (3, 7, 7, 512), (1, 9, 7, 64),
+    (1, 64, 64, 256),  # the shape of tests/bitpack_test.cpp:38-60
+])
+def test_pack_mat(dab, shape):
+    x = special_floats(shape, 1)
+    got = host_u(dab.pack_mat(dev_f(x)))
+    want = np.stack([orc.pack_mat(img) for img in x])
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 4, 5), (2, 128, 7, 9), (1, 512, 56, 56), (3, 192, 1, 1)])
+def test_bitpack_nchw(dab, shape):
+    x = special_floats(shape, 2)
+    got = host_u(dab.bitpack_nchw(dev_f(x)))
+    want = np.stack([orc.pack_nchw(img) for img in x])
+    np.testing.assert_array_equal(got, want)
+    # and it is pack_mat of the NHWC permutation
+    nhwc = np.ascontiguousarray(np.transpose(x, (0, 2, 3, 1)))
+    np.testing.assert_array_equal(got, host_u(dab.pack_mat(dev_f(nhwc))))
+
+
+def test_pack_mat_rejects_bad_channels(dab):
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        dab.pack_mat(torch.zeros((1, 2, 2, 100), device="cuda"))
+
+
+@pytest.mark.parametrize("n,h,w,cw,ph,pw", [(1, 4, 6, 2, 1, 2), (3, 7, 7, 8, 1, 1), (1, 5, 5, 1, 0, 0)])
+def test_pad_bit(dab, n, h, w, cw, ph, pw):
+    x = rng(3).integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    got = host_u(dab.pad(dev_u(x), ph, pw))
+    want = np.stack([orc.pad_bit(img, ph, pw) for img in x])
+    np.testing.assert_array_equal(got, want)
+
+
+# ---------------------------------------------------------------- fused_binarize_im2col
+@pytest.mark.parametrize("n,h,w,c,k,pad,stride,dil", [
+    (1, 8, 8, 128, 3, 1, 1, 1), (2, 8, 8, 64, 3, 1, 2, 1), (1, 7, 9, 192, 3, 1, 1, 1), (1, 6, 6, 128, 5, 2, 2, 1),
+    (2, 5, 5, 3, 3, 1, 1, 1), (1, 4, 4, 100, 1, 0, 1, 1), (1, 10, 10, 64, 3, 2, 1, 2), (1, 28, 28, 128, 3, 1, 1, 1),
+    (1, 14, 14, 256, 3, 1, 2, 1), (2, 7, 7, 512, 3, 1, 1, 1), (1, 3, 3, 128, 3, 0, 2, 1),
+])
+def test_fused_binarize_im2col(dab, n, h, w, c, k, pad, stride, dil):
+    x = special_floats((n, h, w, c), 4)
+    got = host_u(dab.fused_binarize_im2col(dev_f(x), k, k, pad, pad, stride, stride, dil, dil))
+    want = np.concatenate([orc.fused_binarize_im2col(img, k, k, pad, pad, stride, stride, dil, dil) for img in x])
+    np.testing.assert_array_equal(got, want)
+
+
+def test_fused_binarize_im2col_size_limit(dab):
+    with pytest.raises(RuntimeError, match="smaller than 60000"):
+        dab.fused_binarize_im2col(torch.zeros((1, 1, 1, 60000), device="cuda"), 1, 1, 0, 0, 1, 1)
+
+
+# ---------------------------------------------------------------- bgemm
+@pytest.mark.parametrize("m,n,k", [
+    (159, 253, 68),  # tests/bgemm_test.cpp:12-27
+    (128, 784, 18), (256, 196, 36), (512, 49, 72),  # tests/bgemm_test.cpp:132-181
+    (33, 17, 10), (8, 64, 1), (16, 1, 9), (5, 70, 3), (1, 1, 1), (64, 130, 8), (72, 65, 25),
+    (512, 3136, 72),  # BASELINE config 2
+])
+def test_bgemm_matches_naive(dab, m, n, k):
+    a = rng(10).integers(0, 2**64, size=(k, m), dtype=np.uint64)
+    b = rng(11).integers(0, 2**64, size=(n, k), dtype=np.uint64)
+    c0 = rng(12).integers(0, 1000, size=(n, m)).astype(np.float32)  # C is accumulated into
+    want = c0.copy()
+    orc.bgemm_naive(m, n, k, a, m, b, k, want, m)
+    c = dev_f(c0)
+    dab.bgemm(m, n, k, dev_u(a), m, dev_u(b), k, c, m)
+    np.testing.assert_array_equal(c.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("m,n,k,lda,ldb,ldc", [(24, 70, 5, 31, 9, 28), (24, 70, 18, 24, 20, 27), (40, 64, 36, 48, 36, 40),
+                                               (7, 9, 3, 8, 4, 11)])
+def test_bgemm_leading_dimensions(dab, m, n, k, lda, ldb, ldc):
+    a = rng(13).integers(0, 2**64, size=(k, lda), dtype=np.uint64)
+    b = rng(14).integers(0, 2**64, size=(n, ldb), dtype=np.uint64)
+    c0 = rng(15).integers(0, 50, size=(n, ldc)).astype(np.float32)
+    want = c0.copy()
+    orc.bgemm_naive(m, n, k, a, lda, b, ldb, want, ldc)
+    c = dev_f(c0)
+    dab.bgemm(m, n, k, dev_u(a), lda, dev_u(b), ldb, c, ldc)
+    np.testing.assert_array_equal(c.cpu().numpy(), want)
+
+
+def test_bgemm_rejects_bad_arguments(dab):
+    a = torch.zeros(16, dtype=torch.int64, device="cuda")
+    c = torch.zeros(16, dtype=torch.float32, device="cuda")
+    with pytest.raises(RuntimeError, match="leading dimension"):
+        dab.bgemm(4, 2, 2, a, 3, a, 2, c, 4)
+    with pytest.raises(RuntimeError):
+        dab.bgemm(0, 2, 2, a, 4, a, 2, c, 4)
+
+
+def test_weight_transpose(dab):
+    w = rng(16).integers(0, 2**64, size=(24, 18), dtype=np.uint64)
+    np.testing.assert_array_equal(host_u(dab.weight_transpose(dev_u(w))), orc.weight_transpose(w))
+
+
+def test_im2col_transpose_bgemm_equals_baseline_bconv(dab):
+    """The chain asserted by tests/bgemm_test.cpp:32-130 (3x3 stride 2 -> 1x1 output; 5x5 pad 2 stride 2)."""
+    for (h, c, cout, k, pad, stride) in [(3, 128, 128, 3, 0, 2), (9, 128, 16, 5, 2, 2)]:
+        x = rng(17).standard_normal((1, h, h, c)).astype(np.float32)
+        wgt = rng(18).integers(0, 2**64, size=(cout, k * k * c // 64), dtype=np.uint64)
+        want = orc.baseline_bconv(orc.pack_mat(x[0]), wgt, k, k, pad, pad, stride, stride)
+        col = dab.fused_binarize_im2col(dev_f(x), k, k, pad, pad, stride, stride)
+        nrow, kk = col.shape
+        c_out = torch.zeros((nrow, cout), dtype=torch.float32, device="cuda")
+        dab.bgemm(cout, nrow, kk, dab.weight_transpose(dev_u(wgt)), cout, col, kk, c_out, cout)
+        np.testing.assert_array_equal(c_out.cpu().numpy().reshape(want.shape), want)
+
+
+# ---------------------------------------------------------------- direct 3x3 bconv
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,pad", [
+    (1, 8, 8, 64, 64, 1, 1), (1, 8, 8, 128, 128, 1, 1), (1, 8, 8, 256, 64, 1, 1), (1, 8, 8, 512, 32, 1, 1),
+    (2, 9, 7, 64, 8, 1, 1), (3, 7, 10, 128, 24, 2, 1), (1, 6, 6, 64, 40, 1, 0), (2, 5, 5, 256, 16, 2, 0),
+    (1, 3, 3, 128, 128, 2, 0),  # 1x1 output
+    (5, 13, 13, 64, 72, 1, 1),  # pixel count not a multiple of 64, channel groups not a multiple of 4
+    (1, 64, 64, 64, 64, 1, 1), (1, 64, 64, 64, 64, 2, 1),  # tests/bconv_test.cpp:164-250
+    (1, 64, 64, 128, 128, 1, 1),  # tests/bconv_test.cpp bconv_test_3x3_128
+    (1, 32, 32, 256, 256, 1, 1), (1, 16, 16, 512, 256, 1, 1), (1, 16, 16, 512, 1024, 2, 1),
+    (1, 56, 56, 64, 64, 1, 1), (1, 28, 28, 128, 128, 1, 1), (1, 14, 14, 256, 256, 1, 1), (1, 7, 7, 512, 512, 1, 1),
+    (1, 56, 56, 64, 128, 2, 1), (1, 28, 28, 128, 256, 2, 1), (1, 14, 14, 256, 512, 2, 1),  # BASELINE config 3, batch 1
+])
+def test_bconv_3x3_matches_baseline_bconv(dab, n, h, w, cin, cout, stride, pad):
+    cw = cin // 64
+    x = rng(20).integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = rng(21).integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    got = dab.bconv_3x3(dev_u(x), dev_u(wgt), stride, pad).cpu().numpy()
+    want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, pad, pad, stride, stride) for img in x])
+    np.testing.assert_array_equal(got, want)
+
+
+def test_bconv_3x3_equals_pad_then_bconv_on_padded(dab):
+    """bconv_3x3(pad(x)) of the reference == the unpadded entry point with pad 1."""
+    x = rng(22).integers(0, 2**64, size=(2, 10, 10, 2), dtype=np.uint64)
+    wgt = rng(23).integers(0, 2**64, size=(16, 18), dtype=np.uint64)
+    a = dab.bconv_3x3(dev_u(x), dev_u(wgt), 1, 1)
+    b = dab.bconv_3x3(dab.pad(dev_u(x), 1, 1), dev_u(wgt), 1, 0)
+    assert torch.equal(a, b)
+    want = np.stack([orc.bconv_3x3_padded(orc.pad_bit(img, 1, 1), wgt, 1) for img in x])
+    np.testing.assert_array_equal(a.cpu().numpy(), want)
+
+
+def test_bconv_3x3_unsupported_and_invalid(dab):
+    from dabnn_amd.capi import DabUnsupported
+    x = torch.zeros((1, 4, 4, 3), dtype=torch.int64, device="cuda")  # 192 channels
+    w = torch.zeros((8, 27), dtype=torch.int64, device="cuda")
+    with pytest.raises(DabUnsupported):
+        dab.bconv_3x3(x, w)
+    x = torch.zeros((1, 4, 4, 1), dtype=torch.int64, device="cuda")
+    with pytest.raises(DabUnsupported):  # cout not a multiple of 8
+        dab.bconv_3x3(x, torch.zeros((5, 9), dtype=torch.int64, device="cuda"))
+    with pytest.raises(RuntimeError, match="smaller than the kernel"):
+        dab.bconv_3x3(torch.zeros((1, 2, 2, 1), dtype=torch.int64, device="cuda"),
+                      torch.zeros((8, 9), dtype=torch.int64, device="cuda"), 1, 0)
+
+
+# ---------------------------------------------------------------- BinConv layer
+@pytest.mark.parametrize("n,h,w,c,cout,k,pad,stride,method", [
+    (1, 56, 56, 64, 64, 3, 1, 1, 0),  # BASELINE config 1
+    (2, 8, 8, 64, 32, 3, 1, 2, 0), (2, 8, 8, 128, 64, 3, 1, 1, 0), (1, 7, 7, 512, 16, 3, 1, 1, 0),
+    (1, 6, 10, 192, 8, 3, 1, 1, 1),  # 192 channels -> im2col + bgemm
+    (2, 9, 9, 128, 16, 5, 2, 2, 1),  # 5x5
+    (1, 6, 6, 256, 32, 1, 0, 1, 1),  # 1x1
+    (1, 6, 6, 64, 12, 1, 0, 1, 1),  # 64 channels, not 3x3: unpadded filters against padded rows
+    (1, 8, 8, 128, 20, 3, 1, 1, 1),  # cout not a multiple of 8 -> bgemm with a ragged last group
+])
+def test_binconv_layer_matches_reference_dispatch(dab, n, h, w, c, cout, k, pad, stride, method):
+    x = rng(30).standard_normal((n, h, w, c)).astype(np.float32)
+    wf = rng(31).standard_normal((cout, k, k, c)).astype(np.float32)
+    wp = orc.pack_weight(wf)
+    layer = dab.BinConv(dev_u(wp), k, k, pad, pad, stride, stride)
+    got = layer(dev_f(x)).cpu().numpy()
+    assert layer.method == method
+    if c == 64 and k != 3:
+        want = np.stack([orc.baseline_bconv(orc.pack_mat(img), wp, k, k, pad, pad, stride, stride) for img in x])
+    else:
+        want = np.stack([orc.binconv_forward(img, wp, k, k, pad, pad, stride, stride)[0] for img in x])
+    np.testing.assert_array_equal(got, want)
+
+
+def test_binconv_config1_k_minus_2cnt(dab):
+    """BASELINE config 1: counts, then K - 2*cnt through the folded affine, vs a float convolution."""
+    r = rng(32)
+    x = r.standard_normal((1, 56, 56, 64)).astype(np.float32)
+    wf = r.standard_normal((64, 3, 3, 64)).astype(np.float32)
+    layer = dab.BinConv(dev_u(orc.pack_weight(wf)), 3, 3, 1, 1, 1, 1)
+    cnt = layer(dev_f(x))
+    a, b = orc.bn_fold(np.ones(64), np.zeros(64), np.zeros(64), np.ones(64), 0.0, 576)  # identity BN after a bconv
+    y = dab.affine_inplace(cnt.clone(), dev_f(a), dev_f(b)).cpu().numpy()[0]
+    xs = torch.from_numpy(np.where(x[0] > 0, 1.0, -1.0)).permute(2, 0, 1)[None]
+    ws = torch.from_numpy(np.where(wf > 0, 1.0, -1.0)).permute(0, 3, 1, 2)
+    conv = torch.nn.functional.conv2d(torch.nn.functional.pad(xs, (1, 1, 1, 1), value=-1.0), ws)[0].permute(1, 2, 0)
+    np.testing.assert_array_equal(y, conv.numpy().astype(np.float32))
+
+
+# ---------------------------------------------------------------- float glue (1e-4 relative)
+RTOL = 1e-4
+
+
+@pytest.mark.parametrize("n,h,c,cout,k,pad,stride,dil,bias", [
+    (1, 4, 2, 2, 3, 1, 1, 1, False), (1, 8, 2, 2, 5, 2, 2, 1, False), (2, 9, 3, 4, 3, 2, 1, 2, True),
+    (1, 32, 3, 64, 7, 3, 2, 1, False), (2, 7, 64, 128, 1, 0, 1, 1, False), (3, 1, 512, 1000, 1, 0, 1, 1, True),
+    (1, 17, 5, 70, 3, 1, 2, 1, True),
+])
+def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
+    r = rng(40)
+    x = r.standard_normal((n, h, h, c)).astype(np.float32)
+    wgt = r.standard_normal((cout, k, k, c)).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32) if bias else None
+    got = dab.fconv(dev_f(x), dev_f(wgt), dev_f(bv) if bias else None, k, k, pad, pad, stride, stride, dil,
+                    dil).cpu().numpy()
+    want = np.stack([orc.fconv(img, wgt, bv, k, k, pad, pad, stride, stride, dil, dil) for img in x])
+    scale = np.abs(want).max()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+
+
+def test_fconv_ramp_cases_of_reference_tests(dab):
+    """tests/fconv_test.cpp:14-41 and :43-70: ramp image and ramp weights, exact in fp32."""
+    for (h, k, pad, stride) in [(4, 3, 1, 1), (8, 5, 2, 2)]:
+        x = np.arange(h * h * 2, dtype=np.float32).reshape(1, h, h, 2)
+        wgt = np.arange(k * k * 2 * 2, dtype=np.float32).reshape(2, k, k, 2)
+        got = dab.fconv(dev_f(x), dev_f(wgt), None, k, k, pad, pad, stride, stride).cpu().numpy()[0]
+        np.testing.assert_array_equal(got, orc.baseline_fconv(x[0], wgt, k, k, pad, pad, stride, stride))
+
+
+def test_affine_add_bit_exact(dab):
+    r = rng(41)
+    x = r.standard_normal((2, 5, 7, 64)).astype(np.float32)
+    a, b = r.standard_normal(64).astype(np.float32), r.standard_normal(64).astype(np.float32)
+    y = r.standard_normal(x.shape).astype(np.float32)
+    got = dab.affine_inplace(dev_f(x), dev_f(a), dev_f(b))
+    want = np.stack([orc.affine_inplace(img.copy(), a, b) for img in x])
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    got2 = dab.add_inplace(got, dev_f(y)).cpu().numpy()
+    np.testing.assert_array_equal(got2, want + y)
+
+
+@pytest.mark.parametrize("n,h,w,c,k,pad,stride", [(1, 8, 8, 4, 2, 0, 2), (2, 7, 7, 512, 7, 0, 1), (1, 9, 6, 4, 3, 1, 2),
+                                                  (1, 112, 112, 64, 3, 1, 2), (2, 56, 56, 64, 2, 0, 2)])
+def test_pools(dab, n, h, w, c, k, pad, stride):
+    x = rng(42).standard_normal((n, h, w, c)).astype(np.float32)
+    avg = dab.ave_pool(dev_f(x), k, k, pad, pad, stride, stride).cpu().numpy()
+    mx = dab.max_pool(dev_f(x), k, k, pad, pad, stride, stride).cpu().numpy()
+    want_avg = np.stack([orc.ave_pool(img, k, k, pad, pad, stride, stride) for img in x])
+    want_max = np.stack([orc.max_pool(img, k, k, pad, pad, stride, stride) for img in x])
+    np.testing.assert_allclose(avg, want_avg, rtol=RTOL, atol=1e-6)
+    np.testing.assert_array_equal(mx, want_max)
