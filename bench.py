@@ -67,17 +67,25 @@ def main():
     def rand_words(*shape):
         return torch.randint(-2**63, 2**63 - 1, shape, dtype=torch.int64, generator=g).cuda()
 
-    def timed(fn, reps):
-        """Average duration of fn() over reps back-to-back launches, HIP events on the launch stream."""
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    def timed(fn, reps, replays=5):
+        """Average GPU duration of fn(): `reps` launches are captured into a HIP graph (so the Python/ctypes call
+        overhead of ~10 us per launch does not throttle short kernels) and the graph is replayed between two
+        events on its launch stream."""
         fn()
         torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(reps):
+                fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(reps):
-            fn()
+        for _ in range(replays):
+            graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / reps
+        return e0.elapsed_time(e1) * 1e-3 / (reps * replays)
 
     # ------------------------------------------------------------ headline: 7 stage shapes at batch 64
     layers = []
@@ -94,11 +102,16 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
+    step_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(step_graph):
+        step()
+    step_graph.replay()
+    torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
     e0.record()
     for _ in range(args.steps):
-        step()
+        step_graph.replay()
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0

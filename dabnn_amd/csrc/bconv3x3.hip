@@ -22,32 +22,48 @@ struct BconvArgs {
     int H, W, OH, OW;
     int cout;
     int stride, pad;
-    int n_groups;  // cout / 8
-    int n_units;   // tiles * n_groups
-    int n_waves;
+    int n_groups;  // cout / Q channel groups per tile
+    int items_per_wave, items_extra;  // split of the work items over the waves
     uint32_t x_bytes;
-    FastDiv div_ow, div_oh;
+    FastDiv div_ow, div_oh, div_groups;
 };
 
 constexpr int kWavesPerBlock = 4;
 
+// Channels per unit for CW words per pixel: units stay near 600 VALU instructions.
+template <int CW>
+struct UnitChannels {
+    static constexpr int value = CW == 8 ? 2 : (CW == 4 ? 4 : 8);
+};
+
+// Work items handed to waves are runs of S units so that a wave's share of a
+// pixel row always starts and ends on a 16-byte boundary (4 channels).
+template <int Q>
+struct ItemUnits {
+    static constexpr int value = Q >= 4 ? 1 : 4 / Q;
+};
+
 template <int CW>
 __global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
+    constexpr int Q = UnitChannels<CW>::value;
+    constexpr int S = ItemUnits<Q>::value;
+    constexpr int WU = 32 / Q;  // units per 32-channel staging window
     __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     unsigned char *stage = stage_all + wib * kStageBytes;
     const int wv = blockIdx.x * kWavesPerBlock + wib;
 
-    int u0, u1;
-    unit_range(wv, p.n_waves, p.n_units, u0, u1);
-    if (u0 >= u1) return;
+    int i0, i1;
+    item_range(wv, p.items_per_wave, p.items_extra, i0, i1);
+    if (i0 >= i1) return;
+    const int u0 = i0 * S, u1 = i1 * S;
 
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
-    int tile = u0 / p.n_groups;
+    int tile = (int)p.div_groups.div((uint32_t)u0);
     int cg = u0 - tile * p.n_groups;
-    int g_lo = cg & 3;
+    int ch_lo = (cg % WU) * Q;  // first staged channel of the current window
     bool need_load = true;
     uint32_t a[K32];
 
@@ -85,16 +101,18 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const Bco
             }
         }
 
-        uint32_t acc[8];
+        uint32_t acc[Q];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) acc[q] = kAccInit;
-        unit_rowmajor<K32>(p.w + (size_t)cg * 8 * (9 * CW), a, acc);
-        stage_put(stage, lane, cg & 3, acc);
+        for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
+        unit_rowmajor<K32, Q>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
+        const int slot = cg % WU;
+        stage_put<Q>(stage, lane, slot * Q, acc);
 
         const bool last_in_tile = cg == p.n_groups - 1;
-        if ((cg & 3) == 3 || last_in_tile || u == u1 - 1) {
-            stage_flush<false>(stage, lane, p.out, p.cout, tile, p.total, (cg & ~3) * 8, g_lo, cg & 3);
-            g_lo = 0;
+        if (slot == WU - 1 || last_in_tile || u == u1 - 1) {
+            stage_flush<false>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
+                               (slot * Q + Q - 1) >> 2);
+            ch_lo = 0;
         }
         if (last_in_tile) {
             cg = 0;
@@ -107,9 +125,18 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const Bco
 }
 
 template <int CW>
-static int launch_bconv3x3(const BconvArgs &args, hipStream_t stream) {
-    hipLaunchKernelGGL(bconv3x3_kernel<CW>, dim3(args.n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream,
-                       args);
+static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
+    constexpr int Q = UnitChannels<CW>::value;
+    constexpr int S = ItemUnits<Q>::value;
+    a.n_groups = a.cout / Q;
+    const long long items = tiles * (a.n_groups / S);
+    if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW>, 64 * kWavesPerBlock);
+    const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock);
+    a.items_per_wave = (int)(items / n_waves);
+    a.items_extra = (int)(items % n_waves);
+    a.div_groups = FastDiv((uint32_t)a.n_groups);
+    hipLaunchKernelGGL(bconv3x3_kernel<CW>, dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }
@@ -140,18 +167,14 @@ extern "C" int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, con
         return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: tensor too large for 32-bit pixel indexing");
     a.total = (int)total;
     a.cout = cout, a.stride = stride, a.pad = pad;
-    a.n_groups = cout / 8;
-    const long long units = ((total + 63) / 64) * a.n_groups;
-    if (units >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    a.n_units = (int)units;
-    a.n_waves = pick_wave_count(a.n_units, 4, kWavesPerBlock);
     a.x_bytes = (uint32_t)x_bytes;
     a.div_ow = FastDiv((uint32_t)a.OW), a.div_oh = FastDiv((uint32_t)a.OH);
+    const long long tiles = (total + 63) / 64;
     hipStream_t s = as_stream(stream);
     switch (cin) {
-        case 64: return launch_bconv3x3<1>(a, s);
-        case 128: return launch_bconv3x3<2>(a, s);
-        case 256: return launch_bconv3x3<4>(a, s);
-        default: return launch_bconv3x3<8>(a, s);
+        case 64: return launch_bconv3x3<1>(a, tiles, s);
+        case 128: return launch_bconv3x3<2>(a, tiles, s);
+        case 256: return launch_bconv3x3<4>(a, tiles, s);
+        default: return launch_bconv3x3<8>(a, tiles, s);
     }
 }

@@ -4,13 +4,22 @@
 //   B(h,j) = b[j*ldb + h]   k x n words, one contiguous K-row per output pixel
 //   C(i,j) = c[j*ldc + i]   m x n floats, i.e. NHWC output
 //
-// A lane owns one column j (output pixel) and holds its K-row in VGPRs; the 8
-// rows i..i+7 of a unit are one 64-byte scalar load per K word, because A is
-// stored channel-minor.  Two variants:
-//   K64R > 0  the whole K-row (K64R words) stays resident across the units of
-//             a tile (the network shapes: 18, 36, 72 words)
-//   K64R == 0 any k: K is walked in chunks of 8 words whose activations are
-//             re-read per unit (they stay in L1/L2), plus a word-by-word tail
+// Mapping: a lane owns one ROW i of A (an output channel).  For a fixed K word
+// the 64 rows of a tile are 512 contiguous bytes of A, so the lane-resident
+// operand is fetched with fully coalesced loads; the K-row of a column j is
+// contiguous in B and wave-uniform, so it comes through scalar loads and
+// enters v_xor_b32 as SGPR operands; and for a fixed column the 64 results are
+// 256 contiguous bytes of C, so the read-modify-write of C is coalesced
+// without any transposition.
+//
+// A unit is 64 rows x Q columns.  Waves own contiguous ranges of units ordered
+// row-tile major, so the A operand is reloaded only when a range crosses into
+// the next row tile.
+//   K64R > 0  k == K64R and ldb == k: the lane keeps its whole A row resident
+//             (the network shapes: 18, 36, 72 words with Q = 8, 4, 2) and the
+//             Q*k words of B of a unit are one contiguous run
+//   K64R == 0 any k, any ldb: K is walked in chunks of 8 words; per chunk the
+//             lane reloads 8 words of A (coalesced, L1/L2 resident)
 #include "xnor_core.h"
 
 namespace dab {
@@ -21,114 +30,150 @@ struct BgemmArgs {
     float *c;
     int m, n, k;
     int lda, ldb, ldc;
-    int n_groups;  // ceil(m / 8)
-    int n_units;
-    int n_waves;
+    int n_runs;  // ceil(n / Q) column runs per row tile
+    int items_per_wave, items_extra;
+    FastDiv div_runs;
 };
 
 constexpr int kGemmWavesPerBlock = 4;
 constexpr int kChunk = 8;  // K words per chunk of the generic variant
 
-// DIRECT: every lane writes its own 8 results with scalar accesses (any ldc,
-// any alignment); otherwise results go through the staging transpose.
-template <int K64R, bool DIRECT>
-__global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_kernel(const BgemmArgs p) {
-    __shared__ __attribute__((aligned(16))) unsigned char stage_all[DIRECT ? 16 : kGemmWavesPerBlock * kStageBytes];
-    const int lane = threadIdx.x & 63;
-    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    unsigned char *stage = stage_all + (DIRECT ? 0 : wib * kStageBytes);
-    const int wv = blockIdx.x * kGemmWavesPerBlock + wib;
-
-    int u0, u1;
-    unit_range(wv, p.n_waves, p.n_units, u0, u1);
-    if (u0 >= u1) return;
-
-    int tile = u0 / p.n_groups;
-    int cg = u0 - tile * p.n_groups;
-    int g_lo = cg & 3;
-    bool need_load = true;
-    constexpr int NA = K64R > 0 ? 2 * K64R : 2 * kChunk;
-    uint32_t act[NA];
-    const uint64_t *brow = nullptr;
-    const uint32_t stride = (uint32_t)p.lda * 8u;
-
-    for (int u = u0; u < u1; ++u) {
-        if (need_load) {
-            need_load = false;
-            int col = tile * 64 + lane;
-            col = col < p.n ? col : p.n - 1;
-            brow = p.b + (size_t)col * p.ldb;
-            if constexpr (K64R > 0) {
+// C(row, j) += counts of a unit.  Columns below j_first belong to the previous
+// (shifted) run and are skipped; the test is wave-uniform.
+template <int Q>
+__device__ __forceinline__ void add_to_c(float *__restrict__ c, int ldc, int row, bool row_ok, int j0, int j_first,
+                                         const uint32_t (&acc)[Q]) {
 #pragma unroll
-                for (int h = 0; h < K64R; ++h) {
-                    const uint64_t v = brow[h];
-                    act[2 * h] = (uint32_t)v, act[2 * h + 1] = (uint32_t)(v >> 32);
-                }
-            }
-        }
-
-        // The last group of a ragged m is shifted back to end at m, so that its
-        // 64-byte weight loads stay inside A; rows below `first` were already
-        // produced by the previous group and are not written again.
-        const int first = cg * 8;
-        const int i0 = first + 8 <= p.m ? first : p.m - 8;
-        const uint64_t *wbase = p.a + i0;
-
-        uint32_t acc[8];
-#pragma unroll
-        for (int q = 0; q < 8; ++q) acc[q] = kAccInit;
-        if constexpr (K64R > 0) {
-            unit_colmajor<K64R>(wbase, stride, act, acc);
-        } else {
-            int h0 = 0;
-            for (; h0 + kChunk <= p.k; h0 += kChunk) {
-#pragma unroll
-                for (int h = 0; h < kChunk; ++h) {
-                    const uint64_t v = brow[h0 + h];
-                    act[2 * h] = (uint32_t)v, act[2 * h + 1] = (uint32_t)(v >> 32);
-                }
-                unit_colmajor<kChunk>(wbase + (size_t)h0 * p.lda, stride, act, acc);
-            }
-            for (; h0 < p.k; ++h0) {
-                const uint64_t v = brow[h0];
-                act[0] = (uint32_t)v, act[1] = (uint32_t)(v >> 32);
-                unit_colmajor<1>(wbase + (size_t)h0 * p.lda, stride, act, acc);
-            }
-        }
-
-        const bool last_in_tile = cg == p.n_groups - 1;
-        const bool ragged = i0 != first;
-        if (DIRECT || ragged) {
-            const int col = tile * 64 + lane;
-            if (col < p.n) {
-                float *crow = p.c + (size_t)col * p.ldc;
-#pragma unroll
-                for (int q = 0; q < 8; ++q)
-                    if (i0 + q >= first) crow[i0 + q] += __uint_as_float(acc[q]) - kAccBias;
-            }
-        } else {
-            stage_put(stage, lane, cg & 3, acc);
-        }
-        if (!DIRECT) {
-            // a ragged last group is never staged: flush what precedes it in the window
-            const int g_hi = ragged ? (cg & 3) - 1 : (cg & 3);
-            if (((cg & 3) == 3 || last_in_tile || u == u1 - 1)) {
-                if (g_hi >= g_lo) stage_flush<true>(stage, lane, p.c, p.ldc, tile, p.n, (cg & ~3) * 8, g_lo, g_hi);
-                g_lo = 0;
-            }
-        }
-        if (last_in_tile) {
-            cg = 0;
-            ++tile;
-            need_load = true;
-        } else {
-            ++cg;
+    for (int q = 0; q < Q; ++q) {
+        const int j = j0 + q;
+        if (j >= j_first && row_ok) {
+            float *d = c + (size_t)j * ldc + row;
+            *d += __uint_as_float(acc[q]) - kAccBias;
         }
     }
 }
 
-// One thread per output element; for m < 8, where the 8-row units do not apply.
-__global__ void bgemm_small_m_kernel(const BgemmArgs p) {
+template <int K64R, int Q>
+__global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_resident_kernel(const BgemmArgs p) {
+    constexpr int K32 = 2 * K64R;
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wv = blockIdx.x * kGemmWavesPerBlock + wib;
+    int i0, i1;
+    item_range(wv, p.items_per_wave, p.items_extra, i0, i1);
+    if (i0 >= i1) return;
+
+    int mt = (int)p.div_runs.div((uint32_t)i0);
+    int run = i0 - mt * p.n_runs;
+    bool need_load = true;
+    uint32_t w[K32];
+    int row = 0;
+    bool row_ok = false;
+    for (int it = i0; it < i1; ++it) {
+        if (need_load) {
+            need_load = false;
+            row = mt * 64 + lane;
+            row_ok = row < p.m;
+            const uint64_t *col = p.a + (row_ok ? row : p.m - 1);
+#pragma unroll
+            for (int h = 0; h < K64R; ++h) {
+                const uint64_t v = col[(size_t)h * p.lda];
+                w[2 * h] = (uint32_t)v, w[2 * h + 1] = (uint32_t)(v >> 32);
+            }
+        }
+        // the last run of a ragged n is shifted back so its scalar loads stay inside B
+        const int j_first = run * Q;
+        const int j0 = j_first + Q <= p.n ? j_first : p.n - Q;
+        uint32_t acc[Q];
+#pragma unroll
+        for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
+        unit_rowmajor<K32, Q>(p.b + (size_t)j0 * K64R, w, acc);
+        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
+        if (++run == p.n_runs) {
+            run = 0;
+            ++mt;
+            need_load = true;
+        }
+    }
+}
+
+// Any k and ldb; Q = 8 columns per unit, two columns per scalar-load batch.
+__global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_chunked_kernel(const BgemmArgs p) {
+    constexpr int Q = 8;
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wv = blockIdx.x * kGemmWavesPerBlock + wib;
+    int i0, i1;
+    item_range(wv, p.items_per_wave, p.items_extra, i0, i1);
+    if (i0 >= i1) return;
+
+    int mt = (int)p.div_runs.div((uint32_t)i0);
+    int run = i0 - mt * p.n_runs;
+    for (int it = i0; it < i1; ++it) {
+        const int row = mt * 64 + lane;
+        const bool row_ok = row < p.m;
+        const uint64_t *acol = p.a + (row_ok ? row : p.m - 1);
+        const int j_first = run * Q;
+        const int j0 = j_first + Q <= p.n ? j_first : p.n - Q;
+        uint32_t acc[Q];
+#pragma unroll
+        for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
+
+        int h0 = 0;
+        for (; h0 + kChunk <= p.k; h0 += kChunk) {
+            uint32_t w[2 * kChunk];
+#pragma unroll
+            for (int h = 0; h < kChunk; ++h) {
+                const uint64_t v = acol[(size_t)(h0 + h) * p.lda];
+                w[2 * h] = (uint32_t)v, w[2 * h + 1] = (uint32_t)(v >> 32);
+            }
+            // column j0+q contributes the 16 dwords b[(j0+q)*ldb + h0 .. +8)
+            const uint64_t *bbase = p.b + (size_t)j0 * p.ldb + h0;
+            const uint32_t bstride = (uint32_t)p.ldb * 8u;
+            u32x16 buf[2][2];
+            sload_off<16>(buf[0][0], bbase, 0u);
+            sload_off<16>(buf[0][1], bbase, bstride);
+            swait(buf[0][0]);
+            swait(buf[0][1]);
+            uint32_t off = bstride;
+            static_for<Q / 2>([&](auto s_) {
+                constexpr int s = s_;
+                if constexpr (s + 1 < Q / 2) {
+                    off += bstride;
+                    sload_off<16>(buf[(s + 1) & 1][0], bbase, off);
+                    off += bstride;
+                    sload_off<16>(buf[(s + 1) & 1][1], bbase, off);
+                }
+                static_for<2>([&](auto c_) {
+                    static_for<kChunk>([&](auto h_) {
+                        xp2(acc[2 * s + c_], buf[s & 1][c_][2 * h_], buf[s & 1][c_][2 * h_ + 1], w[2 * h_], w[2 * h_ + 1]);
+                    });
+                });
+                if constexpr (s + 1 < Q / 2) {
+                    swait(buf[(s + 1) & 1][0]);
+                    swait(buf[(s + 1) & 1][1]);
+                }
+            });
+        }
+        for (; h0 < p.k; ++h0) {  // K tail, one word at a time
+            const uint64_t v = acol[(size_t)h0 * p.lda];
+            const uint32_t wlo = (uint32_t)v, whi = (uint32_t)(v >> 32);
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const uint64_t bw = p.b[(size_t)(j0 + q) * p.ldb + h0];  // wave-uniform address
+                acc[q] += __builtin_popcount(wlo ^ (uint32_t)bw) + __builtin_popcount(whi ^ (uint32_t)(bw >> 32));
+            }
+        }
+        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
+        if (++run == p.n_runs) {
+            run = 0;
+            ++mt;
+        }
+    }
+}
+
+// One thread per output element; for n < 8, where the column runs do not apply.
+__global__ void bgemm_small_n_kernel(const BgemmArgs p) {
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (long long)p.m * p.n) return;
     const int i = (int)(idx % p.m);
@@ -138,10 +183,25 @@ __global__ void bgemm_small_m_kernel(const BgemmArgs p) {
     p.c[(size_t)j * p.ldc + i] += (float)cnt;
 }
 
-template <int K64R, bool DIRECT>
-static int launch_bgemm(const BgemmArgs &args, hipStream_t stream) {
-    hipLaunchKernelGGL((bgemm_kernel<K64R, DIRECT>), dim3(args.n_waves / kGemmWavesPerBlock),
-                       dim3(64 * kGemmWavesPerBlock), 0, stream, args);
+template <int Q, class Kernel>
+static bool plan_items(BgemmArgs &g, Kernel kernel, int &n_waves) {
+    static const int blocks_per_cu = resident_blocks_per_cu(kernel, 64 * kGemmWavesPerBlock);
+    g.n_runs = (g.n + Q - 1) / Q;
+    const long long items = (((long long)g.m + 63) / 64) * g.n_runs;
+    if (items >= (1ll << 31)) return false;
+    n_waves = pick_wave_count((int)items, blocks_per_cu, kGemmWavesPerBlock);
+    g.items_per_wave = (int)(items / n_waves);
+    g.items_extra = (int)(items % n_waves);
+    g.div_runs = FastDiv((uint32_t)g.n_runs);
+    return true;
+}
+
+template <int K64R, int Q>
+static int launch_resident(BgemmArgs &g, hipStream_t stream) {
+    int n_waves = 0;
+    if (!plan_items<Q>(g, bgemm_resident_kernel<K64R, Q>, n_waves)) return fail(DAB_EUNSUPPORTED, "dab_bgemm: too many work units");
+    hipLaunchKernelGGL((bgemm_resident_kernel<K64R, Q>), dim3(n_waves / kGemmWavesPerBlock), dim3(64 * kGemmWavesPerBlock), 0,
+                       stream, g);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }
@@ -159,30 +219,30 @@ extern "C" int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const 
                     (reinterpret_cast<uintptr_t>(c) & 3) == 0,
                 "dab_bgemm: misaligned pointer");
     if ((long long)k * 64 > kMaxCount) return fail(DAB_EUNSUPPORTED, "dab_bgemm: k %d words exceeds the exact-count range", k);
-    if ((long long)lda * 8 * k >= (1ll << 32)) return fail(DAB_EUNSUPPORTED, "dab_bgemm: A larger than 4 GiB");
+    if ((long long)ldb * 8 * 8 >= (1ll << 32)) return fail(DAB_EUNSUPPORTED, "dab_bgemm: ldb too large");
 
     BgemmArgs g;
     g.a = a, g.b = b, g.c = c;
     g.m = m, g.n = n, g.k = k;
     g.lda = lda, g.ldb = ldb, g.ldc = ldc;
     hipStream_t s = as_stream(stream);
-    if (m < 8) {
+    if (n < 8) {
         const long long total = (long long)m * n;
-        hipLaunchKernelGGL(bgemm_small_m_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g);
+        hipLaunchKernelGGL(bgemm_small_n_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g);
         DAB_LAUNCH_CHECK();
         return DAB_OK;
     }
-    g.n_groups = (m + 7) / 8;
-    const long long units = (((long long)n + 63) / 64) * g.n_groups;
-    if (units >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_bgemm: too many work units");
-    g.n_units = (int)units;
-    g.n_waves = pick_wave_count(g.n_units, 4, kGemmWavesPerBlock);
-    const bool direct = (ldc % 4 != 0) || (reinterpret_cast<uintptr_t>(c) & 15) != 0;
-    if (direct) return launch_bgemm<0, true>(g, s);
-    switch (k) {
-        case 18: return launch_bgemm<18, false>(g, s);
-        case 36: return launch_bgemm<36, false>(g, s);
-        case 72: return launch_bgemm<72, false>(g, s);
-        default: return launch_bgemm<0, false>(g, s);
+    if (ldb == k) {
+        switch (k) {
+            case 18: return launch_resident<18, 8>(g, s);
+            case 36: return launch_resident<36, 4>(g, s);
+            case 72: return launch_resident<72, 2>(g, s);
+            default: break;
+        }
     }
+    int n_waves = 0;
+    if (!plan_items<8>(g, bgemm_chunked_kernel, n_waves)) return fail(DAB_EUNSUPPORTED, "dab_bgemm: too many work units");
+    hipLaunchKernelGGL(bgemm_chunked_kernel, dim3(n_waves / kGemmWavesPerBlock), dim3(64 * kGemmWavesPerBlock), 0, s, g);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
 }

@@ -74,6 +74,7 @@ struct FastDiv {
 // ---------------------------------------------------------------- buffer resources
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
 
 // Raw buffer descriptor over [p, p + bytes): loads with an offset at or beyond

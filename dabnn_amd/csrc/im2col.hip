@@ -6,9 +6,9 @@
 //
 // A wave produces one output word per compare: lane l looks at element
 // 64*wi + l of the row and the lane mask of (value > 0) is the word.  When c
-// is a multiple of 64 a word never straddles two taps, so tap position and
-// bounds test are wave-uniform (scalar) and the 64 lanes read 256 contiguous
-// bytes.  The general path resolves tap and channel per lane.
+// is a multiple of 64 a word never straddles two taps, so the 64 lanes read
+// 256 contiguous bytes of one tap.  The general path resolves tap and channel
+// per lane.
 // HBM-bound on paper (each input float is needed kh*kw times but comes from
 // L2 after the first touch): 4 bytes per input element read, 8 bytes per
 // output word written.
@@ -30,8 +30,53 @@ struct Im2colArgs {
 
 constexpr int kIm2colWavesPerBlock = 4;
 
-template <bool ALIGNED64>
-__global__ __launch_bounds__(64 * kIm2colWavesPerBlock) void fused_binarize_im2col_kernel(const Im2colArgs p) {
+// c % 64 == 0.  Lane l first decodes output word g0 + l of the chunk (row ->
+// image/oy/ox, word -> tap/channel word, bounds test) with ordinary vector
+// arithmetic, 64 words at once; the 64 element offsets are then broadcast one
+// by one (v_readlane) and every word becomes one coalesced 256-byte load, one
+// compare and a select into the owning lane.  All 64 loads are independent.
+__global__ __launch_bounds__(64 * kIm2colWavesPerBlock) void fused_binarize_im2col_aligned_kernel(const Im2colArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long wave = (long long)blockIdx.x * kIm2colWavesPerBlock + wib;
+    const long long n_chunks = (p.n_words + 63) / 64;
+    const long long stride = (long long)gridDim.x * kIm2colWavesPerBlock;
+    const int cw = p.c >> 6;
+    for (long long chunk = wave; chunk < n_chunks; chunk += stride) {
+        const long long g0 = chunk * 64;
+        const uint32_t g = (uint32_t)(g0 + lane);
+        bool ok = (long long)g < p.n_words;
+        const uint32_t row = p.div_row_words.div(ok ? g : 0u);
+        const int wi = (ok ? g : 0u) - row * p.row_words;
+        const uint32_t t = p.div_ow.div(row);
+        const int ox = row - t * p.ow;
+        const uint32_t img = p.div_oh.div(t);
+        const int oy = t - img * p.oh;
+        const uint32_t tap = p.div_cw.div((uint32_t)wi);  // >= kh*kw for the zero padding word
+        const int k = wi - tap * cw;
+        const uint32_t a = p.div_kw.div(tap);
+        const int b = tap - a * p.kw;
+        const int y = oy * p.stride_h - p.pad_h + (int)a * p.dil_h;
+        const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
+        ok = ok && (int)tap < p.kh * p.kw && y >= 0 && y < p.h && xx >= 0 && xx < p.w;
+        // element offset of the word's first float (numel < 2^31 checked on the host); 0 when masked
+        const uint32_t off = ok ? (((img * p.h + y) * p.w + xx) * p.c + k * 64) : 0u;
+        const uint64_t okmask = __ballot(ok);
+        uint64_t mine = 0;
+#pragma unroll 16
+        for (int i = 0; i < 64; ++i) {
+            const uint32_t o = __builtin_amdgcn_readlane(off, i);
+            const float v = p.x[o + lane];
+            uint64_t word = __ballot(v > 0.0f);
+            word = ((okmask >> i) & 1) ? word : 0ull;
+            mine = (lane == i) ? word : mine;
+        }
+        if (g0 + lane < p.n_words) p.col[g0 + lane] = mine;
+    }
+}
+
+// Any c: tap and channel are resolved per lane for every word.
+__global__ __launch_bounds__(64 * kIm2colWavesPerBlock) void fused_binarize_im2col_generic_kernel(const Im2colArgs p) {
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const long long wave = (long long)blockIdx.x * kIm2colWavesPerBlock + wib;
@@ -49,28 +94,16 @@ __global__ __launch_bounds__(64 * kIm2colWavesPerBlock) void fused_binarize_im2c
             const int ox = row - t * p.ow;
             const uint32_t img = p.div_oh.div(t);
             const int oy = t - img * p.oh;
+            const int e = wi * 64 + lane;
             float v = 0.0f;
-            if constexpr (ALIGNED64) {
-                const int cw = p.c >> 6;
-                const uint32_t tap = p.div_cw.div((uint32_t)wi);  // >= kh*kw for the zero padding word
-                const int k = wi - tap * cw;
+            if (e < p.len) {
+                const uint32_t tap = p.div_c.div((uint32_t)e);
+                const int ch = e - tap * p.c;
                 const uint32_t a = p.div_kw.div(tap);
                 const int b = tap - a * p.kw;
                 const int y = oy * p.stride_h - p.pad_h + (int)a * p.dil_h;
                 const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
-                if ((int)tap < p.kh * p.kw && y >= 0 && y < p.h && xx >= 0 && xx < p.w)
-                    v = p.x[(((size_t)img * p.h + y) * p.w + xx) * p.c + k * 64 + lane];
-            } else {
-                const int e = wi * 64 + lane;
-                if (e < p.len) {
-                    const uint32_t tap = p.div_c.div((uint32_t)e);
-                    const int ch = e - tap * p.c;
-                    const uint32_t a = p.div_kw.div(tap);
-                    const int b = tap - a * p.kw;
-                    const int y = oy * p.stride_h - p.pad_h + (int)a * p.dil_h;
-                    const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
-                    if (y >= 0 && y < p.h && xx >= 0 && xx < p.w) v = p.x[(((size_t)img * p.h + y) * p.w + xx) * p.c + ch];
-                }
+                if (y >= 0 && y < p.h && xx >= 0 && xx < p.w) v = p.x[(((size_t)img * p.h + y) * p.w + xx) * p.c + ch];
             }
             const uint64_t word = __ballot(v > 0.0f);
             mine = (lane == i) ? word : mine;
@@ -103,6 +136,7 @@ extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, in
     a.row_words = dab_col_row_words(kh, kw, c);
     a.n_words = (long long)n * a.oh * a.ow * a.row_words;
     if (a.n_words >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_fused_binarize_im2col: more than 2^31 output words");
+    if ((long long)n * h * w * c >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_fused_binarize_im2col: more than 2^31 input elements");
     a.div_row_words = FastDiv((uint32_t)a.row_words);
     a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
     a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv((uint32_t)kw);
@@ -112,10 +146,10 @@ extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, in
     const long long cap = (long long)simd_count() * 8;
     if (blocks > cap) blocks = cap;
     if (c % 64 == 0)
-        hipLaunchKernelGGL(fused_binarize_im2col_kernel<true>, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock), 0,
+        hipLaunchKernelGGL(fused_binarize_im2col_aligned_kernel, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock), 0,
                            as_stream(stream), a);
     else
-        hipLaunchKernelGGL(fused_binarize_im2col_kernel<false>, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock),
+        hipLaunchKernelGGL(fused_binarize_im2col_generic_kernel, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock),
                            0, as_stream(stream), a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;

@@ -2,9 +2,9 @@
 //
 // Work decomposition shared by both kernels
 // -----------------------------------------
-// A "unit" is 64 output pixels (one per lane of a wave) times 8 output
-// channels.  A lane keeps the packed activations of its pixel in VGPRs for as
-// long as the wave stays on the same 64-pixel tile; the weights of the 8
+// A "unit" is 64 output pixels (one per lane of a wave) times Q output
+// channels (Q = 8, 4 or 2).  A lane keeps the packed activations of its pixel in VGPRs for as
+// long as the wave stays on the same 64-pixel tile; the weights of the Q
 // channels are wave-uniform, so they are fetched with scalar loads
 // (s_load_dwordx16 through the scalar data cache) and enter v_xor_b32 as SGPR
 // operands: no VGPR, no LDS traffic and no per-lane address arithmetic for the
@@ -24,18 +24,42 @@
 
 namespace dab {
 
-// 16 dwords of weights through the scalar cache, immediate byte offset.
-template <int OFF>
-__device__ __forceinline__ void sload16(u32x16 &v, const void *p) {
-    asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(v) : "s"(p), "n"(OFF));
+// N dwords (4, 8 or 16) of weights through the scalar cache.
+template <int N>
+struct SVec;
+template <>
+struct SVec<4> {
+    typedef u32x4 type;
+};
+template <>
+struct SVec<8> {
+    typedef u32x8 type;
+};
+template <>
+struct SVec<16> {
+    typedef u32x16 type;
+};
+
+// Immediate byte offset.
+template <int N, int OFF>
+__device__ __forceinline__ void sload(typename SVec<N>::type &v, const void *p) {
+    if constexpr (N == 16) asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(v) : "s"(p), "n"(OFF));
+    if constexpr (N == 8) asm volatile("s_load_dwordx8 %0, %1, %2" : "=s"(v) : "s"(p), "n"(OFF));
+    if constexpr (N == 4) asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(v) : "s"(p), "n"(OFF));
 }
-// Same with a wave-uniform register byte offset.
-__device__ __forceinline__ void sload16_off(u32x16 &v, const void *p, uint32_t off) {
-    asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(v) : "s"(p), "s"(off));
+// Wave-uniform register byte offset.
+template <int N>
+__device__ __forceinline__ void sload_off(typename SVec<N>::type &v, const void *p, uint32_t off) {
+    if constexpr (N == 16) asm volatile("s_load_dwordx16 %0, %1, %2" : "=s"(v) : "s"(p), "s"(off));
+    if constexpr (N == 8) asm volatile("s_load_dwordx8 %0, %1, %2" : "=s"(v) : "s"(p), "s"(off));
+    if constexpr (N == 4) asm volatile("s_load_dwordx4 %0, %1, %2" : "=s"(v) : "s"(p), "s"(off));
 }
 // Scalar loads return out of order: the only usable wait is "all of them".
 // Tying the vector to the statement keeps its consumers behind the wait.
-__device__ __forceinline__ void swait(u32x16 &v) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v)); }
+template <class V>
+__device__ __forceinline__ void swait(V &v) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v));
+}
 
 // acc += popcount(w0 ^ a0) + popcount(w1 ^ a1), weights in SGPRs.
 __device__ __forceinline__ void xp2(uint32_t &acc, uint32_t w0, uint32_t w1, uint32_t a0, uint32_t a1) {
@@ -57,47 +81,74 @@ constexpr float kAccBias = 8388608.0f;
 constexpr int kMaxCount = (1 << 23) - 1;
 
 // ---------------------------------------------------------------- unit bodies
+// A unit is 64 pixels x Q channels, Q in {8, 4, 2}.  Small Q keeps the unit
+// short when the channel count is large: the tail of a launch is one unit
+// executed by a lone wave, and a lone wave issues one VALU instruction per
+// ~6 cycles, so a unit should stay near 600 instructions.
 
-// 8 channels whose K32 weight dwords each lie contiguously ([channel][K32],
-// the reference's weight layout): the 8*K32 dwords are K32/2 vectors of 16.
-template <int K32>
-__device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[8]) {
-    constexpr int NV = K32 / 2;
-    static_assert(K32 % 2 == 0, "a dword pair never straddles two channels");
-    u32x16 buf[2];
-    sload16<0>(buf[0], wbase);
-    swait(buf[0]);
-    static_for<NV>([&](auto j_) {
+// Q channels whose K32 weight dwords each lie contiguously ([channel][K32],
+// the reference's weight layout): Q*K32 dwords read as vectors of 16 (or 8).
+template <int K32, int Q>
+__device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[Q]) {
+    constexpr int D = Q * K32;
+    constexpr int VW = D % 16 == 0 ? 16 : 8;
+    constexpr int NV = D / VW;
+    // Vectors per wait.  A wait can only be "all outstanding scalar loads", so
+    // the latency cover of a batch is the vector work of the previous one: two
+    // vectors (64 vector instructions) ride out a scalar-cache miss to L2.
+    constexpr int BV = (NV % 2 == 0 && VW == 16) ? 2 : 1;
+    constexpr int NB = NV / BV;
+    static_assert(K32 % 2 == 0 && D % VW == 0, "a dword pair never straddles two channels");
+    typename SVec<VW>::type buf[2][BV];
+    static_for<BV>([&](auto b_) { sload<VW, b_ * VW * 4>(buf[0][b_], wbase); });
+    static_for<BV>([&](auto b_) { swait(buf[0][b_]); });
+    static_for<NB>([&](auto j_) {
         constexpr int j = j_;
-        if constexpr (j + 1 < NV) sload16<(j + 1) * 64>(buf[(j + 1) & 1], wbase);
-        static_for<8>([&](auto e_) {
-            constexpr int d = j * 16 + e_ * 2;  // dword index within the 8-channel block
-            constexpr int q = d / K32, k = d % K32;
-            xp2(acc[q], buf[j & 1][e_ * 2], buf[j & 1][e_ * 2 + 1], a[k], a[k + 1]);
+        if constexpr (j + 1 < NB)
+            static_for<BV>([&](auto b_) { sload<VW, ((j + 1) * BV + b_) * VW * 4>(buf[(j + 1) & 1][b_], wbase); });
+        static_for<BV>([&](auto b_) {
+            static_for<VW / 2>([&](auto e_) {
+                constexpr int d = (j * BV + b_) * VW + e_ * 2;  // dword index within the Q-channel block
+                constexpr int q = d / K32, k = d % K32;
+                xp2(acc[q], buf[j & 1][b_][e_ * 2], buf[j & 1][b_][e_ * 2 + 1], a[k], a[k + 1]);
+            });
         });
-        if constexpr (j + 1 < NV) swait(buf[(j + 1) & 1]);
+        if constexpr (j + 1 < NB) static_for<BV>([&](auto b_) { swait(buf[(j + 1) & 1][b_]); });
     });
 }
 
-// 8 channels stored channel-minor ([k word][channel], bgemm's column-major A):
-// vector h holds word h of channels 0..7; consecutive words are `stride`
-// bytes apart.
-template <int K64>
-__device__ __forceinline__ void unit_colmajor(const void *wbase, uint32_t stride, const uint32_t *a, uint32_t (&acc)[8]) {
-    u32x16 buf[2];
-    sload16<0>(buf[0], wbase);
-    swait(buf[0]);
+// Q channels stored channel-minor ([k word][channel], bgemm's column-major A):
+// one scalar load holds word h of channels 0..Q-1; consecutive words are
+// `stride` bytes apart.  Loads are issued in batches of B = 8/Q words (16
+// dwords per batch, like unit_rowmajor) so that each wait is covered by 32
+// vector instructions.
+template <int K64, int Q>
+__device__ __forceinline__ void unit_colmajor(const void *wbase, uint32_t stride, const uint32_t *a, uint32_t (&acc)[Q]) {
+    constexpr int VW = 2 * Q;
+    constexpr int B = (K64 % (8 / Q) == 0) ? 8 / Q : 1;
+    constexpr int NB = K64 / B;
+    typename SVec<VW>::type buf[2][B];
     uint32_t off = 0;
-    static_for<K64>([&](auto h_) {
-        constexpr int h = h_;
-        if constexpr (h + 1 < K64) {
-            off += stride;
-            sload16_off(buf[(h + 1) & 1], wbase, off);
+    static_for<B>([&](auto b_) {
+        sload_off<VW>(buf[0][b_], wbase, off);
+        off += stride;
+    });
+    static_for<B>([&](auto b_) { swait(buf[0][b_]); });
+    static_for<NB>([&](auto j_) {
+        constexpr int j = j_;
+        if constexpr (j + 1 < NB) {
+            static_for<B>([&](auto b_) {
+                sload_off<VW>(buf[(j + 1) & 1][b_], wbase, off);
+                off += stride;
+            });
         }
-        static_for<8>([&](auto q_) {
-            xp2(acc[q_], buf[h & 1][q_ * 2], buf[h & 1][q_ * 2 + 1], a[2 * h], a[2 * h + 1]);
+        static_for<B>([&](auto b_) {
+            constexpr int h = j * B + b_;
+            static_for<Q>([&](auto q_) {
+                xp2(acc[q_], buf[j & 1][b_][q_ * 2], buf[j & 1][b_][q_ * 2 + 1], a[2 * h], a[2 * h + 1]);
+            });
         });
-        if constexpr (h + 1 < K64) swait(buf[(h + 1) & 1]);
+        if constexpr (j + 1 < NB) static_for<B>([&](auto b_) { swait(buf[(j + 1) & 1][b_]); });
     });
 }
 
@@ -109,22 +160,30 @@ __device__ __forceinline__ void unit_colmajor(const void *wbase, uint32_t stride
 constexpr int kStageRow = 144;                // 32 channels * 4 B + 16 B pad: conflict-free b128 access
 constexpr int kStageBytes = 64 * kStageRow;   // per wave
 
-__device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int slot, const uint32_t (&acc)[8]) {
-    float4 *dst = reinterpret_cast<float4 *>(stage + lane * kStageRow + slot * 32);
-    dst[0] = make_float4(__uint_as_float(acc[0]) - kAccBias, __uint_as_float(acc[1]) - kAccBias,
-                         __uint_as_float(acc[2]) - kAccBias, __uint_as_float(acc[3]) - kAccBias);
-    dst[1] = make_float4(__uint_as_float(acc[4]) - kAccBias, __uint_as_float(acc[5]) - kAccBias,
-                         __uint_as_float(acc[6]) - kAccBias, __uint_as_float(acc[7]) - kAccBias);
+// Parks the Q results of a lane at channel offset ch_off (multiple of Q) of its row.
+template <int Q>
+__device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch_off, const uint32_t (&acc)[Q]) {
+    float f[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) f[q] = __uint_as_float(acc[q]) - kAccBias;
+    unsigned char *row = stage + lane * kStageRow + ch_off * 4;
+    if constexpr (Q == 2) {
+        *reinterpret_cast<float2 *>(row) = make_float2(f[0], f[1]);
+    } else {
+#pragma unroll
+        for (int q = 0; q < Q; q += 4) *reinterpret_cast<float4 *>(row + q * 4) = make_float4(f[q], f[q + 1], f[q + 2], f[q + 3]);
+    }
 }
 
-// Writes staged channel groups [g_lo, g_hi] of the 32-channel window that
-// starts at channel cbase.  out is [pixel][ld] floats; pixels >= total are
-// skipped.  ACCUM adds to what out already holds (bgemm's C +=).
+// Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
+// 32-channel window that starts at channel cbase.  out is [pixel][ld] floats;
+// pixels >= total are skipped.  ACCUM adds to what out already holds
+// (bgemm's C +=).
 template <bool ACCUM>
 __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
-                                            int tile, int total, int cbase, int g_lo, int g_hi) {
+                                            int tile, int total, int cbase, int p_lo, int p_hi) {
     __builtin_amdgcn_wave_barrier();
-    const int np = 2 * (g_hi - g_lo + 1);  // 16-byte parts per pixel row
+    const int np = p_hi - p_lo + 1;  // 16-byte parts per pixel row
     if (np == 8 && (tile + 1) * 64 <= total) {
         const int pr0 = lane >> 3, part = lane & 7;
         const unsigned char *src = stage + pr0 * kStageRow + part * 16;
@@ -144,7 +203,7 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
         for (int i = 0; i < np; ++i) {
             const int c = lane + 64 * i;
             const int pr = (c * magic) >> 16;
-            const int part = 2 * g_lo + (c - pr * np);
+            const int part = p_lo + (c - pr * np);
             const int pix = tile * 64 + pr;
             if (pix < total) {
                 float4 v = *reinterpret_cast<const float4 *>(stage + pr * kStageRow + part * 16);
@@ -160,16 +219,27 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
     __builtin_amdgcn_wave_barrier();
 }
 
-// Contiguous unit range [u0, u1) of wave `wv` out of `n_waves`.
-__device__ __forceinline__ void unit_range(int wv, int n_waves, int n_units, int &u0, int &u1) {
-    u0 = (int)(((long long)wv * n_units) / n_waves);
-    u1 = (int)(((long long)(wv + 1) * n_units) / n_waves);
+// Contiguous item range [i0, i1) of wave `wv`: every wave gets `per` items and
+// the first `extra` waves one more (per = n_items / n_waves, extra = the rest).
+__device__ __forceinline__ void item_range(int wv, int per, int extra, int &i0, int &i1) {
+    i0 = wv * per + (wv < extra ? wv : extra);
+    i1 = i0 + per + (wv < extra ? 1 : 0);
 }
 
-// Host side: how many waves to launch for n_units units.
-inline int pick_wave_count(int n_units, int waves_per_simd, int waves_per_block) {
-    long long w = (long long)simd_count() * waves_per_simd;
-    if (w > n_units) w = n_units;
+// Host side: how many waves to launch for n_items work items.  All of them
+// must be resident at once (a second round of waves would start when the
+// first is nearly done and unbalance the SIMDs), so the count follows the
+// kernel's real occupancy: blocks per CU as limited by VGPRs and LDS.
+template <class Kernel>
+inline int resident_blocks_per_cu(Kernel kernel, int block_threads) {
+    int blocks = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, kernel, block_threads, 0) != hipSuccess || blocks < 1) blocks = 1;
+    return blocks;
+}
+
+inline int pick_wave_count(int n_items, int blocks_per_cu, int waves_per_block) {
+    long long w = (long long)(simd_count() / 4) * blocks_per_cu * waves_per_block;
+    if (w > n_items) w = n_items;
     if (w < 1) w = 1;
     return (int)((w + waves_per_block - 1) / waves_per_block * waves_per_block);
 }
