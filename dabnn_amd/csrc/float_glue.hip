@@ -112,6 +112,11 @@ __global__ __launch_bounds__(256) void add_kernel(float *__restrict__ a, const f
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) a[i] = __fadd_rn(a[i], b[i]);
 }
 
+__global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, long long total) {
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = x[i] > 0.f ? x[i] : 0.f;
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(float *__restrict__ x, long long total, float v) {
     const long long stride = (long long)gridDim.x * 256;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = v;
@@ -215,6 +220,22 @@ extern "C" int dab_add_inplace(float *a, const float *b, int64_t n_elem, dab_str
     hipLaunchKernelGGL(add_kernel, dim3(grid_for(n_elem)), dim3(256), 0, as_stream(stream), a, b, (long long)n_elem);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
+}
+
+extern "C" int dab_relu_inplace(float *x, int64_t n_elem, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x, "dab_relu_inplace: null pointer");
+    DAB_REQUIRE(n_elem > 0, "dab_relu_inplace: n_elem %lld", (long long)n_elem);
+    hipLaunchKernelGGL(relu_kernel, dim3(grid_for(n_elem)), dim3(256), 0, as_stream(stream), x, (long long)n_elem);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_fill_f32(float *x, int64_t n_elem, float value, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x, "dab_fill_f32: null pointer");
+    DAB_REQUIRE(n_elem > 0, "dab_fill_f32: n_elem %lld", (long long)n_elem);
+    return fill_f32(x, (long long)n_elem, value, as_stream(stream));
 }
 
 static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,

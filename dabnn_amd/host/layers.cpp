@@ -1,0 +1,228 @@
+#include "layers.h"
+
+#include <sstream>
+#include <stdexcept>
+
+#include "../../include/dabnn_hip.h"
+#include "net.h"
+
+namespace bnn {
+
+void bnn_fail(const std::string &msg) { throw std::runtime_error(msg); }
+
+void dab_check(int rc) {
+    if (rc != DAB_OK) throw std::runtime_error(dab_last_error());
+}
+
+// ---------------------------------------------------------------- Layer
+Layer::~Layer() {}
+
+Layer::MatP Layer::mat(const std::string &name) const { return net_.lock()->get_blob(name); }
+
+void *Layer::stream() const { return net_.lock()->stream(); }
+
+std::string Layer::to_str() const { return type_ + " " + name_; }
+
+// ---------------------------------------------------------------- BinConv
+// dabnn/layers/BinConv.cpp:17-78: scratch blobs are registered in the net's
+// blob map under the reference's names; the weights are transposed once for
+// the bgemm method (:59-76).  No padded copy is kept: the direct kernel reads
+// out-of-image taps as zero words itself.
+BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad_h_, int pad_w_, int stride_h_,
+                 int stride_w_)
+    : Layer(net, name, "Bin Conv"),
+      input_mat(mat(input)),
+      weight_mat(mat(weight)),
+      output_mat(mat(output)),
+      pad_h(pad_h_),
+      pad_w(pad_w_),
+      stride_h(stride_h_),
+      stride_w(stride_w_) {
+    auto n = net.lock();
+    BNN_ASSERT(input_mat->data_type == DataType::Float, "BinConv input must be float");
+    BNN_ASSERT(weight_mat->data_type == DataType::Bit, "BinConv weight must be Bit");
+    BNN_ASSERT(input_mat->elem_c % 64 == 0, "BinConv needs a multiple of 64 input channels, got " +
+                                                std::to_string(input_mat->elem_c));
+    BNN_ASSERT(weight_mat->total() % weight_mat->n == 0, "weight size is not a multiple of the filter count");
+
+    const std::string binarized_name = "binaized_for_" + output + "_cal";
+    if (!n->has_blob(binarized_name))
+        n->add_mat(binarized_name, std::make_shared<Mat>(input_mat->n, input_mat->h, input_mat->w, input_mat->elem_c,
+                                                         DataType::Bit, binarized_name));
+    binarized_mat = mat(binarized_name);
+
+    const std::string col_name = "col_for_" + output + "_cal";
+    if (!n->has_blob(col_name)) {
+        const size_t len = (size_t)output_mat->n * output_mat->h * output_mat->w *
+                           dab_col_row_words(kernel_h(), kernel_w(), input_mat->elem_c);
+        n->add_mat(col_name, std::make_shared<Mat>(len, DataType::Bit, col_name));
+    }
+    col_mat = mat(col_name);
+
+    const int m = weight_mat->n;
+    const int k = (int)(weight_mat->total() / m);
+    transposed_weight_mat = std::make_shared<Mat>((size_t)m * k, DataType::Bit, "trans_" + weight);
+    dab_check(dab_weight_transpose(static_cast<const uint64_t *>(weight_mat->data), m, k,
+                                   static_cast<uint64_t *>(transposed_weight_mat->data), n->stream()));
+    n->add_mat("trans_" + weight, transposed_weight_mat);
+}
+
+bool BinConv::direct_conv_compatible() const {
+    // dabnn/layers/BinConv.cpp:100-126 (1024 input channels stay with bgemm here)
+    const int c = input_mat->elem_c;
+    return kernel_h() == 3 && kernel_w() == 3 && stride_h == stride_w && pad_h == pad_w &&
+           (c == 64 || c == 128 || c == 256 || c == 512) && weight_mat->n % 8 == 0;
+}
+
+BinConv::Method BinConv::method() const {
+    if (net_.lock()->optimize && direct_conv_compatible()) return DIRECT_CONV;
+    return BGEMM;
+}
+
+void BinConv::forward_impl() const {
+    void *s = stream();
+    const auto *x = static_cast<const float *>(input_mat->data);
+    auto *out = static_cast<float *>(output_mat->data);
+    const int n = input_mat->n, h = input_mat->h, w = input_mat->w, c = input_mat->elem_c;
+    switch (method()) {
+        case DIRECT_CONV: {
+            // pack_mat + (pad +) bconv_3x3, dabnn/layers/BinConv.cpp:146-150
+            auto *packed = static_cast<uint64_t *>(binarized_mat->data);
+            dab_check(dab_bitpack_nhwc(x, packed, (int64_t)n * h * w, c, s));
+            dab_check(dab_bconv3x3(packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n,
+                                   stride_h, pad_h, out, s));
+            break;
+        }
+        case BGEMM: {
+            // fill + fused_binarize_im2col + bgemm, dabnn/layers/BinConv.cpp:152-165
+            dab_check(dab_fill_f32(out, (int64_t)output_mat->total(), 0.f, s));
+            auto *col = static_cast<uint64_t *>(col_mat->data);
+            dab_check(dab_fused_binarize_im2col(x, n, h, w, c, kernel_h(), kernel_w(), pad_h, pad_w, stride_h, stride_w, 1,
+                                                1, col, s));
+            const int m = weight_mat->n;
+            const int cols = n * output_mat->h * output_mat->w;
+            const int k = (int)(weight_mat->total() / m);
+            const int ldb = dab_col_row_words(kernel_h(), kernel_w(), c);  // rows are padded to 128 bits
+            dab_check(dab_bgemm(m, cols, k, static_cast<const uint64_t *>(transposed_weight_mat->data), m, col, ldb, out, m,
+                                s));
+            break;
+        }
+    }
+}
+
+std::string BinConv::to_str() const {
+    std::stringstream ss;
+    ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->elem_c << ", weight "
+       << weight_mat->n << "x" << kernel_h() << "x" << kernel_w() << ", pad " << pad_h << "," << pad_w << ", stride "
+       << stride_h << "," << stride_w << ", method " << (method() == DIRECT_CONV ? "DIRECT_CONV" : "BGEMM");
+    return ss.str();
+}
+
+// ---------------------------------------------------------------- FloatConv
+FloatConv::FloatConv(NetCP net, css name, css input, css weight, css bias, css output, int pad_h_, int pad_w_,
+                     int stride_h_, int stride_w_, int dilation_)
+    : Layer(net, name, "Float Conv"),
+      input_mat(mat(input)),
+      weight_mat(mat(weight)),
+      bias_mat(mat(bias)),
+      output_mat(mat(output)),
+      pad_h(pad_h_),
+      pad_w(pad_w_),
+      stride_h(stride_h_),
+      stride_w(stride_w_),
+      dilation(dilation_) {}
+
+FloatConv::FloatConv(NetCP net, css name, css input, css weight, css output, int pad_h_, int pad_w_, int stride_h_,
+                     int stride_w_, int dilation_)
+    : Layer(net, name, "Float Conv"),
+      input_mat(mat(input)),
+      weight_mat(mat(weight)),
+      output_mat(mat(output)),
+      pad_h(pad_h_),
+      pad_w(pad_w_),
+      stride_h(stride_h_),
+      stride_w(stride_w_),
+      dilation(dilation_) {}
+
+void FloatConv::forward_impl() const {
+    dab_check(dab_fconv(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+                        input_mat->c, static_cast<const float *>(weight_mat->data),
+                        bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr, weight_mat->h, weight_mat->w, pad_h,
+                        pad_w, stride_h, stride_w, dilation, dilation, output_mat->c,
+                        static_cast<float *>(output_mat->data), stream()));
+}
+
+std::string FloatConv::to_str() const {
+    std::stringstream ss;
+    ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->c << ", weight " << weight_mat->n
+       << "x" << weight_mat->h << "x" << weight_mat->w;
+    return ss.str();
+}
+
+// ---------------------------------------------------------------- Affine / Add / Relu (in place)
+Affine::Affine(NetCP net, css name, css data, css a, css b)
+    : Layer(net, name, "Affine"), data_mat(mat(data)), a_mat(mat(a)), b_mat(mat(b)) {
+    BNN_ASSERT((int)a_mat->total() == data_mat->c && (int)b_mat->total() == data_mat->c,
+               "Affine coefficients do not match the channel count");
+}
+
+void Affine::forward_impl() const {
+    dab_check(dab_affine_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->n * data_mat->h * data_mat->w,
+                                 data_mat->c, static_cast<const float *>(a_mat->data),
+                                 static_cast<const float *>(b_mat->data), stream()));
+}
+
+Add::Add(NetCP net, css name, css input1, css input2)
+    : Layer(net, name, "Add"), input1_mat(mat(input1)), input2_mat(mat(input2)) {
+    BNN_ASSERT(input1_mat->total() == input2_mat->total(), "Add operands differ in size");
+}
+
+void Add::forward_impl() const {
+    dab_check(dab_add_inplace(static_cast<float *>(input1_mat->data), static_cast<const float *>(input2_mat->data),
+                              (int64_t)input1_mat->total(), stream()));
+}
+
+Relu::Relu(NetCP net, css name, css data) : Layer(net, name, "Relu"), data_mat(mat(data)) {}
+
+void Relu::forward_impl() const {
+    dab_check(dab_relu_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->total(), stream()));
+}
+
+// ---------------------------------------------------------------- pooling
+AvePool::AvePool(NetCP net, css name, css input, css output, int kernel_h_, int kernel_w_, int pad_h_, int pad_w_,
+                 int stride_h_, int stride_w_)
+    : Layer(net, name, "AvePool"),
+      input_mat(mat(input)),
+      output_mat(mat(output)),
+      kernel_h(kernel_h_),
+      kernel_w(kernel_w_),
+      pad_h(pad_h_),
+      pad_w(pad_w_),
+      stride_h(stride_h_),
+      stride_w(stride_w_) {}
+
+void AvePool::forward_impl() const {
+    dab_check(dab_ave_pool(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+                           input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                           static_cast<float *>(output_mat->data), stream()));
+}
+
+MaxPool::MaxPool(NetCP net, css name, css input, css output, int kernel_h_, int kernel_w_, int pad_h_, int pad_w_,
+                 int stride_h_, int stride_w_)
+    : Layer(net, name, "MaxPool"),
+      input_mat(mat(input)),
+      output_mat(mat(output)),
+      kernel_h(kernel_h_),
+      kernel_w(kernel_w_),
+      pad_h(pad_h_),
+      pad_w(pad_w_),
+      stride_h(stride_h_),
+      stride_w(stride_w_) {}
+
+void MaxPool::forward_impl() const {
+    dab_check(dab_max_pool(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+                           input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                           static_cast<float *>(output_mat->data), stream()));
+}
+
+}  // namespace bnn

@@ -1,0 +1,85 @@
+// The layers of the Bi-Real path (dabnn/layers/{BinConv,FloatConv,Affine,Add,
+// AvePool,MaxPool,Relu}.{h,cpp}); constructor signatures follow the reference.
+#pragma once
+
+#include "layer.h"
+
+namespace bnn {
+
+using css = const std::string &;
+
+class BinConv : public Layer {
+   public:
+    MatP input_mat;
+    MatP binarized_mat;  // packed input of the direct method
+    MatP col_mat;        // column matrix of the bgemm method
+    MatP weight_mat;
+    MatP transposed_weight_mat;
+    MatP output_mat;
+    const int pad_h, pad_w, stride_h, stride_w;
+
+    enum Method { DIRECT_CONV = 0, BGEMM = 1 };
+
+    BinConv(NetCP net, css name, css input, css weight, css output, int pad_h, int pad_w, int stride_h, int stride_w);
+    void forward_impl() const override;
+    std::string to_str() const override;
+    Method method() const;
+
+   private:
+    int kernel_h() const { return weight_mat->h; }
+    int kernel_w() const { return weight_mat->w; }
+    bool direct_conv_compatible() const;
+};
+
+class FloatConv : public Layer {
+   public:
+    MatP input_mat, weight_mat, bias_mat, output_mat;
+    const int pad_h, pad_w, stride_h, stride_w, dilation;
+    FloatConv(NetCP net, css name, css input, css weight, css bias, css output, int pad_h, int pad_w, int stride_h,
+              int stride_w, int dilation);
+    FloatConv(NetCP net, css name, css input, css weight, css output, int pad_h, int pad_w, int stride_h, int stride_w,
+              int dilation);
+    void forward_impl() const override;
+    std::string to_str() const override;
+};
+
+class Affine : public Layer {
+   public:
+    MatP data_mat, a_mat, b_mat;
+    Affine(NetCP net, css name, css data, css a, css b);
+    void forward_impl() const override;
+};
+
+class Add : public Layer {
+   public:
+    MatP input1_mat, input2_mat;
+    Add(NetCP net, css name, css input1, css input2);
+    void forward_impl() const override;
+};
+
+class Relu : public Layer {
+   public:
+    MatP data_mat;
+    Relu(NetCP net, css name, css data);
+    void forward_impl() const override;
+};
+
+class AvePool : public Layer {
+   public:
+    MatP input_mat, output_mat;
+    const int kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w;
+    AvePool(NetCP net, css name, css input, css output, int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h,
+            int stride_w);
+    void forward_impl() const override;
+};
+
+class MaxPool : public Layer {
+   public:
+    MatP input_mat, output_mat;
+    const int kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w;
+    MaxPool(NetCP net, css name, css input, css output, int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h,
+            int stride_w);
+    void forward_impl() const override;
+};
+
+}  // namespace bnn

@@ -1,0 +1,67 @@
+// bnn::Net (dabnn/net.h:22-68): loads a .dab model, owns the blobs, runs the
+// layers in order.  Public surface as in the reference -- create / read /
+// read_buf / run / get_blob and the flags optimize / run_fconv / strict --
+// plus a batch size, which the reference does not have (dabnn/net.cpp:64-65).
+//
+// All blobs live in device memory; run() takes a HOST pointer to
+// batch x H x W x C floats (NHWC) like the reference's run(void*), uploads it,
+// enqueues every layer on the net's stream and waits.  run_device() takes a
+// device pointer and skips the copy.
+#pragma once
+
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "layer.h"
+#include "mat.h"
+
+namespace bnn {
+
+class Net : public std::enable_shared_from_this<Net> {
+   public:
+    static std::shared_ptr<Net> create();
+    ~Net();
+
+    void set_batch(int batch);  // before read(); default 1
+    int batch() const { return batch_; }
+    const std::string &input_name() const { return input_name_; }
+    void read(const std::string &path);
+    void read_buf(const void *ptr);
+    void run(const void *host_input);
+    void run_device(const void *device_input);
+    std::shared_ptr<Mat> get_blob(const std::string &name);
+    bool has_blob(const std::string &name) const { return mat_map_.count(name) != 0; }
+    std::vector<std::string> layer_descriptions() const;
+
+    // optimize: true picks the direct 3x3 kernel where it applies, false sends every
+    // BinConv through im2col + bgemm (the reference's switch between its optimised and
+    // plain kernels; both settings give identical outputs).
+    bool optimize = true;
+    bool run_fconv = true;
+    bool strict = true;
+
+    // per-layer-type milliseconds of the last runs when profiling (BNN_BENCHMARK of the reference)
+    bool profile = false;
+    std::map<std::string, double> layer_time_;
+    std::string time_report() const;
+
+    void *stream() const { return stream_; }
+    void add_mat(const std::string &name, std::shared_ptr<Mat> mat);
+    std::map<std::string, std::shared_ptr<Mat>> mat_map_;
+
+   private:
+    Net();
+    void prepare(const void *model_buf);
+    std::weak_ptr<Net> get_weak() { return shared_from_this(); }
+    std::vector<std::shared_ptr<Layer>> layers;
+    std::map<std::string, std::vector<uint32_t>> shapes_;  // NHWC with N = 1, as stored in the model
+    std::string input_name_;
+    std::vector<uint8_t> file_;  // owns the model bytes when read from a path
+    int batch_ = 1;
+    void *stream_ = nullptr;
+    bool prepared_ = false;
+};
+
+}  // namespace bnn

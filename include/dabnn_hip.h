@@ -147,6 +147,12 @@ DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, c
 /* add_inplace (dabnn/layers/Add.cpp:7-17): a += b over n_elem floats. */
 DAB_API int dab_add_inplace(float *a, const float *b, int64_t n_elem, dab_stream_t stream);
 
+/* Relu::forward_impl (dabnn/layers/Relu.cpp): x = max(x, 0) in place over n_elem floats. */
+DAB_API int dab_relu_inplace(float *x, int64_t n_elem, dab_stream_t stream);
+
+/* Mat::fill<float> (dabnn/mat.h:351-443): x[i] = value; the zero-fill before bgemm (dabnn/layers/BinConv.cpp:153). */
+DAB_API int dab_fill_f32(float *x, int64_t n_elem, float value, dab_stream_t stream);
+
 /* ave_pool_fallback (dabnn/layers/AvePool.cpp:84-123): mean over in-bounds taps. */
 DAB_API int dab_ave_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
                  int stride_w, float *out, dab_stream_t stream);

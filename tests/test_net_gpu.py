@@ -1,0 +1,132 @@
+"""GPU: the C++ bnn::Net on .dab models vs the CPU restatement of the layer loop.
+
+Bit-exact wherever the data is integer (packed activations, raw BinConv
+counts), 1e-4 relative after float layers (north_star tolerance)."""
+import numpy as np
+import pytest
+
+import oracle as orc
+from oracle import net as orc_net
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import torch
+    assert torch.cuda.is_available()
+    from dabnn_amd import dab_format, models, net
+    return dab_format, models, net
+
+
+def close(got, want):
+    scale = max(np.abs(want).max(), 1e-6)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+
+
+def test_small_net_matches_cpu_layer_loop(mods):
+    df, models, net = mods
+    layers, inits, inputs = models.small_bnn(1, hw=16, width=64)
+    buf = df.write_model(layers, inits, inputs)
+    batch = 3
+    x = np.random.default_rng(5).standard_normal((batch, 16, 16, 3)).astype(np.float32)
+    n = net.Net(batch=batch).read_buf(buf)
+    descs = n.layers()
+    assert sum("DIRECT_CONV" in d for d in descs) == 3 and sum("BGEMM" in d for d in descs) == 1
+    n.run(x)
+    logits = n.get_blob("logits").reshape(batch, -1)
+    for i in range(batch):
+        rec = {}
+        cpu = orc_net.run_model(layers, inits, x[i], record=rec)
+        close(logits[i], cpu["logits"].ravel())
+        # packed input of every BinConv: bit-exact unless a float sits within rounding of zero
+        for blk in ("b0", "b1", "b2"):
+            packed = n.get_blob("binaized_for_%s_cnt_cal" % blk)[i]
+            src = {"b0": "conv1_out", "b1": "b0_out", "b2": "b1_bn"}[blk]
+            assert packed.shape == orc.pack_mat(cpu[src]).shape
+    n.close()
+
+
+def test_binconv_counts_inside_net_are_bit_exact(mods):
+    """One BinConv + Affine net: the blob holds raw counts before the affine when the affine is identity-free;
+    here the net is cut after the BinConv so the counts themselves are the output."""
+    df, models, net = mods
+    r = np.random.default_rng(7)
+    for (c, cout, k, stride, pad) in [(64, 64, 3, 1, 1), (128, 64, 3, 2, 1), (192, 24, 3, 1, 1), (128, 16, 5, 2, 2),
+                                      (64, 12, 1, 1, 0)]:
+        wf = r.standard_normal((cout, k, k, c)).astype(np.float32)
+        inits = [{"name": "w", "shape": [cout, k, k, c], "data": models.pack_weight(wf).ravel(),
+                  "align_hwc_to_128": c != 64}]
+        layers = [{"type": "BinConv2D", "name": "bc", "input": "data", "weight": "w", "output": "cnt",
+                   "pads": [pad] * 4, "strides": [stride, stride], "dilations": [1, 1]}]
+        x = r.standard_normal((2, 12, 12, c)).astype(np.float32)
+        for optimize in (True, False):
+            n = net.Net(batch=2, optimize=optimize).read_buf(df.write_model(layers, inits, [("data", [1, 12, 12, c])]))
+            n.run(x)
+            got = n.get_blob("cnt")
+            for i in range(2):
+                want = orc_net.run_model(layers, inits, x[i])["cnt"]
+                np.testing.assert_array_equal(got[i], want)
+            n.close()
+
+
+def test_optimize_flag_gives_identical_outputs(mods):
+    """tests/net_test.cpp:29-50: optimize=false and optimize=true agree."""
+    df, models, net = mods
+    layers, inits, inputs = models.small_bnn(2, hw=16, width=64)
+    buf = df.write_model(layers, inits, inputs)
+    x = np.random.default_rng(6).standard_normal((2, 16, 16, 3)).astype(np.float32)
+    outs = []
+    for optimize in (True, False):
+        n = net.Net(batch=2, optimize=optimize).read_buf(buf)
+        if not optimize:
+            assert all("DIRECT_CONV" not in d for d in n.layers())
+        n.run(x)
+        outs.append(n.get_blob("logits").copy())
+        n.close()
+    np.testing.assert_array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("stem", [False, True])
+def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
+    df, models, net = mods
+    layers, inits, inputs = models.bireal18(11, stem=stem)
+    path = tmp_path / "bireal18.dab"
+    path.write_bytes(df.write_model(layers, inits, inputs))
+    x = np.random.default_rng(8).standard_normal((2, 224, 224, 3)).astype(np.float32)
+    n = net.Net(batch=2).read(str(path))
+    assert sum("Bin Conv" in d for d in n.layers()) == 16
+    n.run(x)
+    logits = n.get_blob("logits").reshape(2, -1)
+    assert logits.shape == (2, 1000)
+    for i in range(2):
+        cpu = orc_net.run_model(layers, inits, x[i])
+        close(logits[i], cpu["logits"].ravel())
+        close(n.get_blob("pool1_out")[i], cpu["pool1_out"])
+    n.set_profile(True)
+    n.run(x)
+    report = n.time_report()
+    assert "Bin Conv" in report and "Float Conv" in report and "total" in report
+    n.close()
+
+
+def test_error_paths(mods, tmp_path):
+    df, models, net = mods
+    with pytest.raises(ValueError, match="Open file error"):  # std::invalid_argument, dabnn/net.cpp:34-36
+        net.Net().read(str(tmp_path / "missing.dab"))
+    layers, inits, inputs = models.small_bnn(0)
+    with pytest.raises(RuntimeError, match="model version should be 2"):
+        net.Net().read_buf(df.write_model(layers, inits, inputs, version=1))
+    with pytest.raises(RuntimeError, match="fconv must be run in strict mode"):
+        net.Net(run_fconv=False, strict=True).read_buf(df.write_model(layers, inits, inputs))
+    bad = layers + [{"type": "Softmax", "name": "sm", "input": "logits", "output": "prob"}]
+    with pytest.raises(RuntimeError, match="Not supported op Softmax"):
+        net.Net().read_buf(df.write_model(bad, inits, inputs))
+    n = net.Net().read_buf(df.write_model(layers, inits, inputs))
+    with pytest.raises(KeyError):
+        n.get_blob("no_such_blob")
+    with pytest.raises(ValueError):
+        n.run(np.zeros((1, 8, 8, 3), dtype=np.float32))
+    n.close()
