@@ -13,6 +13,7 @@ from .ops import (  # noqa: F401
     affine_inplace,
     ave_pool,
     bconv_3x3,
+    bconv_3x3_affine_add,
     bgemm,
     bitpack_nchw,
     col_row_words,

@@ -24,6 +24,9 @@ class DabUnsupported(DabError):
 
 
 def _load():
+    # torch ships its own copy of the HIP runtime.  Import it first so that this library binds to the runtime that
+    # owns torch's device context; two runtimes in one process do not see each other's devices.
+    import torch  # noqa: F401
     if not os.path.exists(LIB_PATH):
         raise ImportError(
             "%s is missing: build it with `make -C dabnn_amd/csrc` (or __graft_entry__.build()); "
@@ -48,6 +51,7 @@ SIGNATURES = {
     "dab_bgemm": (_i, [_i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp]),
     "dab_weight_transpose": (_i, [_vp, _i, _i, _vp, _vp]),
     "dab_bconv3x3": (_i, [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp]),
+    "dab_bconv3x3_affine_add": (_i, [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dab_binconv_workspace_bytes": (_sz, [_i] * 10),
     "dab_binconv_forward": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 8 + [_vp, _vp, _sz, ctypes.POINTER(_i), _vp]),
     "dab_fconv": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 9 + [_vp, _vp]),

@@ -26,6 +26,10 @@ struct BconvArgs {
     int items_per_wave, items_extra;  // split of the work items over the waves
     uint32_t x_bytes;
     FastDiv div_ow, div_oh, div_groups;
+    // fused epilogue (FUSED kernels only): out = a*cnt + b (+ shortcut)
+    const float *epi_a;
+    const float *epi_b;
+    const float *epi_shortcut;
 };
 
 constexpr int kWavesPerBlock = 4;
@@ -43,8 +47,10 @@ struct ItemUnits {
     static constexpr int value = Q >= 4 ? 1 : 4 / Q;
 };
 
-template <int CW>
-__global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const BconvArgs p) {
+// The second launch bound asks the register allocator for 3 resident waves per SIMD at 512 channels
+// (144 of the 512/3 = 168 available VGPRs hold the activations), 4 otherwise (the staging buffers allow no more).
+template <int CW, bool FUSED>
+__global__ __launch_bounds__(64 * kWavesPerBlock, CW == 8 ? 3 : 4) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
     constexpr int Q = UnitChannels<CW>::value;
     constexpr int S = ItemUnits<Q>::value;
@@ -104,14 +110,21 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const Bco
         uint32_t acc[Q];
 #pragma unroll
         for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
-        unit_rowmajor<K32, Q>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
+        unit_rowmajor<K32, Q, (CW >= 2 ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
         const int slot = cg % WU;
         stage_put<Q>(stage, lane, slot * Q, acc);
 
         const bool last_in_tile = cg == p.n_groups - 1;
         if (slot == WU - 1 || last_in_tile || u == u1 - 1) {
-            stage_flush<false>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
-                               (slot * Q + Q - 1) >> 2);
+            if constexpr (FUSED) {
+                EpiAffineAdd epi;
+                epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+                stage_flush(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
+                            epi);
+            } else {
+                stage_flush(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
+                            EpiStore());
+            }
             ch_lo = 0;
         }
         if (last_in_tile) {
@@ -124,57 +137,86 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void bconv3x3_kernel(const Bco
     }
 }
 
-template <int CW>
+template <int CW, bool FUSED>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW>::value;
     constexpr int S = ItemUnits<Q>::value;
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW>, 64 * kWavesPerBlock);
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, FUSED>, 64 * kWavesPerBlock);
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
     a.div_groups = FastDiv((uint32_t)a.n_groups);
-    hipLaunchKernelGGL(bconv3x3_kernel<CW>, dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
+    hipLaunchKernelGGL((bconv3x3_kernel<CW, FUSED>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }
 
 }  // namespace dab
 
-extern "C" int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
-                            int pad, float *out, dab_stream_t stream) {
+static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
+                         int stride, int pad, const float *a_coef, const float *b_coef, const float *shortcut, bool fused,
+                         float *out, dab_stream_t stream) {
     using namespace dab;
-    DAB_REQUIRE(x && wgt && out, "dab_bconv3x3: null pointer");
-    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0, "dab_bconv3x3: non-positive dimension");
-    DAB_REQUIRE(stride > 0 && pad >= 0, "dab_bconv3x3: stride %d pad %d", stride, pad);
-    DAB_REQUIRE(cin % 64 == 0, "dab_bconv3x3: cin %d is not a multiple of 64", cin);
-    DAB_REQUIRE(h + 2 * pad >= 3 && w + 2 * pad >= 3, "dab_bconv3x3: input smaller than the kernel");
+    DAB_REQUIRE(x && wgt && out, "%s: null pointer", fn);
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0, "%s: non-positive dimension", fn);
+    DAB_REQUIRE(stride > 0 && pad >= 0, "%s: stride %d pad %d", fn, stride, pad);
+    DAB_REQUIRE(cin % 64 == 0, "%s: cin %d is not a multiple of 64", fn, cin);
+    DAB_REQUIRE(h + 2 * pad >= 3 && w + 2 * pad >= 3, "%s: input smaller than the kernel", fn);
     if (!(cin == 64 || cin == 128 || cin == 256 || cin == 512) || cout % 8 != 0)
-        return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: cin %d / cout %d not covered by the direct kernel", cin, cout);
+        return fail(DAB_EUNSUPPORTED, "%s: cin %d / cout %d not covered by the direct kernel", fn, cin, cout);
     DAB_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wgt) & 7) == 0 &&
                     (reinterpret_cast<uintptr_t>(out) & 15) == 0,
-                "dab_bconv3x3: buffers must be 16-byte aligned");
+                "%s: buffers must be 16-byte aligned", fn);
+    if (fused) {
+        DAB_REQUIRE(a_coef && b_coef, "%s: null affine coefficients", fn);
+        DAB_REQUIRE((reinterpret_cast<uintptr_t>(a_coef) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_coef) & 15) == 0 &&
+                        (reinterpret_cast<uintptr_t>(shortcut) & 15) == 0,
+                    "%s: coefficient and shortcut buffers must be 16-byte aligned", fn);
+    }
 
     BconvArgs a;
     a.x = x, a.w = wgt, a.out = out;
+    a.epi_a = a_coef, a.epi_b = b_coef, a.epi_shortcut = shortcut;
     a.H = h, a.W = w;
     a.OH = out_dim(h, pad, 3, 1, stride), a.OW = out_dim(w, pad, 3, 1, stride);
     const long long total = (long long)n * a.OH * a.OW;
     const long long x_bytes = (long long)n * h * w * (cin / 64) * 8;
     if (total >= (1ll << 31) - 64 || x_bytes >= (1ll << 31) || total * cout >= (1ll << 40))
-        return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: tensor too large for 32-bit pixel indexing");
+        return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit pixel indexing", fn);
     a.total = (int)total;
     a.cout = cout, a.stride = stride, a.pad = pad;
     a.x_bytes = (uint32_t)x_bytes;
     a.div_ow = FastDiv((uint32_t)a.OW), a.div_oh = FastDiv((uint32_t)a.OH);
     const long long tiles = (total + 63) / 64;
     hipStream_t s = as_stream(stream);
-    switch (cin) {
-        case 64: return launch_bconv3x3<1>(a, tiles, s);
-        case 128: return launch_bconv3x3<2>(a, tiles, s);
-        case 256: return launch_bconv3x3<4>(a, tiles, s);
-        default: return launch_bconv3x3<8>(a, tiles, s);
+    if (fused) {
+        switch (cin) {
+            case 64: return launch_bconv3x3<1, true>(a, tiles, s);
+            case 128: return launch_bconv3x3<2, true>(a, tiles, s);
+            case 256: return launch_bconv3x3<4, true>(a, tiles, s);
+            default: return launch_bconv3x3<8, true>(a, tiles, s);
+        }
     }
+    switch (cin) {
+        case 64: return launch_bconv3x3<1, false>(a, tiles, s);
+        case 128: return launch_bconv3x3<2, false>(a, tiles, s);
+        case 256: return launch_bconv3x3<4, false>(a, tiles, s);
+        default: return launch_bconv3x3<8, false>(a, tiles, s);
+    }
+}
+
+extern "C" int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
+                            int pad, float *out, dab_stream_t stream) {
+    return bconv3x3_impl("dab_bconv3x3", x, n, h, w, cin, wgt, cout, stride, pad, nullptr, nullptr, nullptr, false, out,
+                         stream);
+}
+
+extern "C" int dab_bconv3x3_affine_add(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
+                                       int stride, int pad, const float *a, const float *b, const float *shortcut,
+                                       float *out, dab_stream_t stream) {
+    return bconv3x3_impl("dab_bconv3x3_affine_add", x, n, h, w, cin, wgt, cout, stride, pad, a, b, shortcut, true, out,
+                         stream);
 }

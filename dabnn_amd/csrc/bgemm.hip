@@ -54,7 +54,7 @@ __device__ __forceinline__ void add_to_c(float *__restrict__ c, int ldc, int row
 }
 
 template <int K64R, int Q>
-__global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_resident_kernel(const BgemmArgs p) {
+__global__ __launch_bounds__(64 * kGemmWavesPerBlock, K64R >= 72 ? 3 : (K64R >= 36 ? 5 : 6)) void bgemm_resident_kernel(const BgemmArgs p) {
     constexpr int K32 = 2 * K64R;
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_resident_kernel
         uint32_t acc[Q];
 #pragma unroll
         for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
-        unit_rowmajor<K32, Q>(p.b + (size_t)j0 * K64R, w, acc);
+        unit_rowmajor<K32, Q, 2>(p.b + (size_t)j0 * K64R, w, acc);  // B streams through the scalar cache: two vectors per wait
         add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
         if (++run == p.n_runs) {
             run = 0;

@@ -88,15 +88,16 @@ constexpr int kMaxCount = (1 << 23) - 1;
 
 // Q channels whose K32 weight dwords each lie contiguously ([channel][K32],
 // the reference's weight layout): Q*K32 dwords read as vectors of 16 (or 8).
-template <int K32, int Q>
+// BV = vectors per wait.  A wait can only be "all outstanding scalar loads",
+// so the latency cover of a batch is the vector work of the previous one: one
+// vector (32 vector instructions) covers a scalar-cache hit, two ride out a
+// miss to L2 (operands too large for the 16 KiB scalar cache).
+template <int K32, int Q, int BV_WANTED = 1>
 __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[Q]) {
     constexpr int D = Q * K32;
     constexpr int VW = D % 16 == 0 ? 16 : 8;
     constexpr int NV = D / VW;
-    // Vectors per wait.  A wait can only be "all outstanding scalar loads", so
-    // the latency cover of a batch is the vector work of the previous one: two
-    // vectors (64 vector instructions) ride out a scalar-cache miss to L2.
-    constexpr int BV = (NV % 2 == 0 && VW == 16) ? 2 : 1;
+    constexpr int BV = (NV % BV_WANTED == 0) ? BV_WANTED : 1;
     constexpr int NB = NV / BV;
     static_assert(K32 % 2 == 0 && D % VW == 0, "a dword pair never straddles two channels");
     typename SVec<VW>::type buf[2][BV];
@@ -175,28 +176,55 @@ __device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch
     }
 }
 
+// What happens to four consecutive channels of one pixel on their way out.
+//   EpiStore      out = cnt                                  (the reference's BinConv output)
+//   EpiAffineAdd  out = a[ch]*cnt + b[ch] (+ shortcut)       (BinConv -> Affine -> Add of a residual block in one
+//                 pass; multiply, add and add are rounded separately, exactly like the three layers)
+struct EpiStore {
+    __device__ __forceinline__ void prepare(int) {}
+    __device__ __forceinline__ float4 operator()(float4 v, const float4 *, size_t) const { return v; }
+};
+struct EpiAffineAdd {
+    const float *a;
+    const float *b;
+    const float *shortcut;  // may be null; same layout as out
+    float4 av, bv;
+    __device__ __forceinline__ void prepare(int ch) {
+        av = *reinterpret_cast<const float4 *>(a + ch);
+        bv = *reinterpret_cast<const float4 *>(b + ch);
+    }
+    __device__ __forceinline__ float4 operator()(float4 v, const float4 *, size_t off) const {
+#pragma clang fp contract(off)
+        float4 r;
+        r.x = av.x * v.x, r.y = av.y * v.y, r.z = av.z * v.z, r.w = av.w * v.w;
+        r.x = r.x + bv.x, r.y = r.y + bv.y, r.z = r.z + bv.z, r.w = r.w + bv.w;
+        if (shortcut) {
+            const float4 sc = *reinterpret_cast<const float4 *>(shortcut + off);
+            r.x = r.x + sc.x, r.y = r.y + sc.y, r.z = r.z + sc.z, r.w = r.w + sc.w;
+        }
+        return r;
+    }
+};
+
 // Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
 // 32-channel window that starts at channel cbase.  out is [pixel][ld] floats;
-// pixels >= total are skipped.  ACCUM adds to what out already holds
-// (bgemm's C +=).
-template <bool ACCUM>
+// pixels >= total are skipped.
+template <class Epi>
 __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
-                                            int tile, int total, int cbase, int p_lo, int p_hi) {
+                                            int tile, int total, int cbase, int p_lo, int p_hi, Epi epi) {
     __builtin_amdgcn_wave_barrier();
     const int np = p_hi - p_lo + 1;  // 16-byte parts per pixel row
     if (np == 8 && (tile + 1) * 64 <= total) {
         const int pr0 = lane >> 3, part = lane & 7;
         const unsigned char *src = stage + pr0 * kStageRow + part * 16;
-        float *dst = out + ((size_t)tile * 64 + pr0) * ld + cbase + part * 4;
+        const size_t off0 = ((size_t)tile * 64 + pr0) * ld + cbase + part * 4;
+        epi.prepare(cbase + part * 4);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float4 v = *reinterpret_cast<const float4 *>(src + i * 8 * kStageRow);
-            float4 *d = reinterpret_cast<float4 *>(dst + (size_t)i * 8 * ld);
-            if (ACCUM) {
-                const float4 o = *d;
-                v.x += o.x, v.y += o.y, v.z += o.z, v.w += o.w;
-            }
-            *d = v;
+            const float4 v = *reinterpret_cast<const float4 *>(src + i * 8 * kStageRow);
+            const size_t off = off0 + (size_t)i * 8 * ld;
+            float4 *d = reinterpret_cast<float4 *>(out + off);
+            *d = epi(v, d, off);
         }
     } else {
         const int magic = (65536 + np - 1) / np;  // c / np for c < 512
@@ -206,13 +234,11 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             const int part = p_lo + (c - pr * np);
             const int pix = tile * 64 + pr;
             if (pix < total) {
-                float4 v = *reinterpret_cast<const float4 *>(stage + pr * kStageRow + part * 16);
-                float4 *d = reinterpret_cast<float4 *>(out + (size_t)pix * ld + cbase + part * 4);
-                if (ACCUM) {
-                    const float4 o = *d;
-                    v.x += o.x, v.y += o.y, v.z += o.z, v.w += o.w;
-                }
-                *d = v;
+                const float4 v = *reinterpret_cast<const float4 *>(stage + pr * kStageRow + part * 16);
+                const size_t off = (size_t)pix * ld + cbase + part * 4;
+                float4 *d = reinterpret_cast<float4 *>(out + off);
+                epi.prepare(cbase + part * 4);
+                *d = epi(v, d, off);
             }
         }
     }

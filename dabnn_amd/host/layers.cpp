@@ -89,8 +89,15 @@ void BinConv::forward_impl() const {
             // pack_mat + (pad +) bconv_3x3, dabnn/layers/BinConv.cpp:146-150
             auto *packed = static_cast<uint64_t *>(binarized_mat->data);
             dab_check(dab_bitpack_nhwc(x, packed, (int64_t)n * h * w, c, s));
-            dab_check(dab_bconv3x3(packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n,
-                                   stride_h, pad_h, out, s));
+            if (fused_a) {
+                dab_check(dab_bconv3x3_affine_add(
+                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n, stride_h, pad_h,
+                    static_cast<const float *>(fused_a->data), static_cast<const float *>(fused_b->data),
+                    fused_shortcut ? static_cast<const float *>(fused_shortcut->data) : nullptr, out, s));
+            } else {
+                dab_check(dab_bconv3x3(packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n,
+                                       stride_h, pad_h, out, s));
+            }
             break;
         }
         case BGEMM: {
@@ -115,6 +122,7 @@ std::string BinConv::to_str() const {
     ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->elem_c << ", weight "
        << weight_mat->n << "x" << kernel_h() << "x" << kernel_w() << ", pad " << pad_h << "," << pad_w << ", stride "
        << stride_h << "," << stride_w << ", method " << (method() == DIRECT_CONV ? "DIRECT_CONV" : "BGEMM");
+    if (fused_a) ss << (fused_shortcut ? " + Affine + Add" : " + Affine");
     return ss.str();
 }
 

@@ -20,6 +20,10 @@ class BinConv : public Layer {
 
     enum Method { DIRECT_CONV = 0, BGEMM = 1 };
 
+    // Set by Net::prepare when the layers that follow are Affine (and Add) on this layer's output and the direct
+    // kernel applies: the three run as one pass with identical results.
+    MatP fused_a, fused_b, fused_shortcut;
+
     BinConv(NetCP net, css name, css input, css weight, css output, int pad_h, int pad_w, int stride_h, int stride_w);
     void forward_impl() const override;
     std::string to_str() const override;

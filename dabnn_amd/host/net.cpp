@@ -78,6 +78,7 @@ Net::Net() {
 }
 
 Net::~Net() {
+    if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
     layers.clear();
     mat_map_.clear();
     if (stream_) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
@@ -274,8 +275,34 @@ void Net::prepare(const void *buf) {
                                          (type >= 0 && type <= PRelu ? kLayerTypeNames[type] : "unknown"));
         }
     }
+    if (optimize) fuse_binconv_epilogues();
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)), "hipStreamSynchronize");
     prepared_ = true;
+}
+
+// BinConv -> Affine (-> Add) on the same blob becomes one pass of the direct kernel.  Blob names and contents after
+// run() are unchanged: the in-place layers wrote into the BinConv output blob anyway.
+void Net::fuse_binconv_epilogues() {
+    std::vector<std::shared_ptr<Layer>> out;
+    for (size_t i = 0; i < layers.size(); ++i) {
+        auto bc = std::dynamic_pointer_cast<BinConv>(layers[i]);
+        auto af = i + 1 < layers.size() ? std::dynamic_pointer_cast<Affine>(layers[i + 1]) : nullptr;
+        if (bc && af && bc->method() == BinConv::DIRECT_CONV && af->data_mat == bc->output_mat && bc->output_mat->c % 4 == 0) {
+            bc->fused_a = af->a_mat;
+            bc->fused_b = af->b_mat;
+            size_t skip = 1;
+            auto ad = i + 2 < layers.size() ? std::dynamic_pointer_cast<Add>(layers[i + 2]) : nullptr;
+            if (ad && ad->input1_mat == bc->output_mat && ad->input2_mat != bc->output_mat) {
+                bc->fused_shortcut = ad->input2_mat;
+                skip = 2;
+            }
+            out.push_back(bc);
+            i += skip;
+        } else {
+            out.push_back(layers[i]);
+        }
+    }
+    layers.swap(out);
 }
 
 void Net::run(const void *host_input) {
@@ -295,7 +322,31 @@ void Net::run_device(const void *device_input) {
         auto in = get_blob(input_name_);
         hip_check(hipMemcpyAsync(in->data, device_input, in->bytes(), hipMemcpyDeviceToDevice, s), "hipMemcpyAsync");
     }
-    for (const auto &layer : layers) layer->forward();
+    if (profile || !use_graph) {
+        for (const auto &layer : layers) layer->forward();
+    } else if (graph_exec_) {
+        hip_check(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_), s), "hipGraphLaunch");
+    } else if (runs_ >= 2) {
+        // capture the kernels of one forward pass; nothing in the layers allocates, synchronises or memsets
+        hipGraph_t graph = nullptr;
+        hip_check(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+        try {
+            for (const auto &layer : layers) layer->forward();
+        } catch (...) {
+            (void)hipStreamEndCapture(s, &graph);
+            if (graph) (void)hipGraphDestroy(graph);
+            throw;
+        }
+        hip_check(hipStreamEndCapture(s, &graph), "hipStreamEndCapture");
+        hipGraphExec_t exec = nullptr;
+        hip_check(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+        (void)hipGraphDestroy(graph);
+        graph_exec_ = exec;
+        hip_check(hipGraphLaunch(exec, s), "hipGraphLaunch");
+    } else {
+        for (const auto &layer : layers) layer->forward();
+    }
+    ++runs_;
     hip_check(hipStreamSynchronize(s), "hipStreamSynchronize");
 }
 

@@ -42,6 +42,11 @@ class Net : public std::enable_shared_from_this<Net> {
     bool run_fconv = true;
     bool strict = true;
 
+    // Replay the layer sequence as one HIP graph from the third run on (the first two run eagerly so that every
+    // kernel has been launched once outside capture).  Launch overhead dominates at batch 1; switch off to
+    // debug or when layers are added between runs.
+    bool use_graph = true;
+
     // per-layer-type milliseconds of the last runs when profiling (BNN_BENCHMARK of the reference)
     bool profile = false;
     std::map<std::string, double> layer_time_;
@@ -54,6 +59,7 @@ class Net : public std::enable_shared_from_this<Net> {
    private:
     Net();
     void prepare(const void *model_buf);
+    void fuse_binconv_epilogues();
     std::weak_ptr<Net> get_weak() { return shared_from_this(); }
     std::vector<std::shared_ptr<Layer>> layers;
     std::map<std::string, std::vector<uint32_t>> shapes_;  // NHWC with N = 1, as stored in the model
@@ -62,6 +68,8 @@ class Net : public std::enable_shared_from_this<Net> {
     int batch_ = 1;
     void *stream_ = nullptr;
     bool prepared_ = false;
+    int runs_ = 0;
+    void *graph_exec_ = nullptr;
 };
 
 }  // namespace bnn

@@ -67,6 +67,10 @@ int dabnet_set_flags(dabnet_t *net, int optimize, int run_fconv, int strict) {
     });
 }
 
+int dabnet_set_use_graph(dabnet_t *net, int on) {
+    return guarded([&] { net->net->use_graph = on != 0; });
+}
+
 int dabnet_set_profile(dabnet_t *net, int on) {
     return guarded([&] {
         net->net->profile = on != 0;

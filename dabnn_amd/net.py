@@ -30,6 +30,7 @@ NET_SIGNATURES = {
     "dabnet_destroy": (None, [_vp]),
     "dabnet_set_batch": (_i, [_vp, _i]),
     "dabnet_set_flags": (_i, [_vp, _i, _i, _i]),
+    "dabnet_set_use_graph": (_i, [_vp, _i]),
     "dabnet_set_profile": (_i, [_vp, _i]),
     "dabnet_time_report": (_cp, [_vp]),
     "dabnet_read_file": (_i, [_vp, _cp]),
@@ -123,6 +124,9 @@ class Net:
         if int(np.prod(shape)) == out.size:
             out = out.reshape(shape)
         return out
+
+    def set_use_graph(self, on=True):
+        _check(hostlib.dabnet_set_use_graph(self._h, int(on)))
 
     def set_profile(self, on=True):
         _check(hostlib.dabnet_set_profile(self._h, int(on)))

@@ -118,6 +118,27 @@ def bconv_3x3(x, weight, stride=1, pad=1):
     return out
 
 
+def bconv_3x3_affine_add(x, weight, a, b, shortcut=None, stride=1, pad=1):
+    """bconv_3x3, affine_inplace and add_inplace of a residual block in one pass: a*cnt + b (+ shortcut)."""
+    _need(x, torch.int64, "x")
+    _need(weight, torch.int64, "weight")
+    _need(a, torch.float32, "a")
+    _need(b, torch.float32, "b")
+    n, h, w, cw = x.shape
+    cout = weight.shape[0]
+    if weight.numel() != cout * 9 * cw or a.numel() != cout or b.numel() != cout:
+        raise capi.DabError(capi.DAB_EINVAL, "bconv_3x3_affine_add: operand sizes do not match")
+    oh, ow = out_dim(h, pad, 3, stride), out_dim(w, pad, 3, stride)
+    out = _empty((n, max(oh, 0), max(ow, 0), cout), torch.float32, x.device)
+    if shortcut is not None:
+        _need(shortcut, torch.float32, "shortcut")
+        if shortcut.shape != out.shape:
+            raise capi.DabError(capi.DAB_EINVAL, "bconv_3x3_affine_add: shortcut shape differs from the output")
+    check(lib.dab_bconv3x3_affine_add(_ptr(x), n, h, w, cw * 64, _ptr(weight), cout, stride, pad, _ptr(a), _ptr(b),
+                                      _ptr(shortcut) if shortcut is not None else None, _ptr(out), _stream()))
+    return out
+
+
 class BinConv:
     """The BinConv layer (dabnn/layers/BinConv.h:9-38, BinConv.cpp:17-191) over a batch.
 

@@ -114,6 +114,19 @@ DAB_API int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const 
                  int pad, float *out, dab_stream_t stream);
 
 /*
+ * dab_bconv3x3 followed in the same pass by the two layers that always follow a
+ * BinConv in a residual block: affine_inplace (dabnn/layers/Affine.cpp:10-23)
+ * and add_inplace (dabnn/layers/Add.cpp:7-17):
+ *   out[p][c] = (a[c] * cnt[p][c] + b[c]) + shortcut[p][c]
+ * with the three operations rounded one by one, so the result equals running
+ * the three reference layers in sequence bit for bit.  shortcut may be NULL
+ * (affine only); it has the layout of out and must not overlap it.
+ */
+DAB_API int dab_bconv3x3_affine_add(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
+                                    int stride, int pad, const float *a, const float *b, const float *shortcut,
+                                    float *out, dab_stream_t stream);
+
+/*
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in

@@ -44,6 +44,8 @@ DABNET_API void dabnet_destroy(dabnet_t *net);
 DABNET_API int dabnet_set_batch(dabnet_t *net, int batch);
 /* The public flags of bnn::Net (dabnn/net.h:59-61); call before reading the model. */
 DABNET_API int dabnet_set_flags(dabnet_t *net, int optimize, int run_fconv, int strict);
+/* Replay the forward pass as one HIP graph from the third run on (default on). */
+DABNET_API int dabnet_set_use_graph(dabnet_t *net, int on);
 /* Per-layer-type timing, the reference's BNN_BENCHMARK build option (dabnn/layer.cpp:17-31). */
 DABNET_API int dabnet_set_profile(dabnet_t *net, int on);
 DABNET_API const char *dabnet_time_report(dabnet_t *net);

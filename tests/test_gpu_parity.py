@@ -192,6 +192,27 @@ def test_bconv_3x3_equals_pad_then_bconv_on_padded(dab):
     np.testing.assert_array_equal(a.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,with_shortcut", [
+    (2, 9, 7, 64, 64, 1, True), (1, 14, 14, 256, 256, 1, True), (3, 8, 8, 128, 24, 2, True), (1, 7, 7, 512, 64, 1, False),
+    (5, 13, 13, 64, 72, 1, True), (1, 56, 56, 64, 64, 1, True),
+])
+def test_bconv_affine_add_equals_three_reference_layers(dab, n, h, w, cin, cout, stride, with_shortcut):
+    r = rng(24)
+    cw = cin // 64
+    x = r.integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, 1, 1, stride, stride) for img in x])
+    sc = r.standard_normal(want.shape).astype(np.float32) if with_shortcut else None
+    for img in want:
+        orc.affine_inplace(img, a, b)
+    if with_shortcut:
+        want = want + sc  # add_inplace: one rounding per element, as numpy
+    got = dab.bconv_3x3_affine_add(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), dev_f(sc) if with_shortcut else None, stride, 1)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
 def test_bconv_3x3_unsupported_and_invalid(dab):
     from dabnn_amd.capi import DabUnsupported
     x = torch.zeros((1, 4, 4, 3), dtype=torch.int64, device="cuda")  # 192 channels

@@ -1,0 +1,118 @@
+"""GPU: BASELINE shapes at full batch size, checked through properties that do
+not need the CPU oracle to chew through billions of bit operations:
+
+* an independent textbook computation on the GPU itself: for +-1 tensors the
+  mismatch count equals (K - conv2d(sign x, sign w, padding value -1)) / 2,
+  with conv2d from torch (exact in fp32: |sums| <= 4608 < 2^24);
+* complement symmetry: cnt(~x, w) + cnt(x, w) == 9*Cin on interior pixels;
+* batch consistency: every image of a batch equals the batch-1 result;
+* bgemm linearity in C: running twice adds the counts twice.
+A sample of outputs is also compared with the CPU oracle.
+"""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+STAGE_SHAPES = [(56, 64, 64, 1), (28, 128, 128, 1), (14, 256, 256, 1), (7, 512, 512, 1), (56, 64, 128, 2),
+                (28, 128, 256, 2), (14, 256, 512, 2)]
+
+
+@pytest.fixture(scope="module")
+def dab():
+    import dabnn_amd
+    assert torch.cuda.is_available()
+    return dabnn_amd
+
+
+def unpack_pm1(words, c):
+    """int64 [..., cw] -> float +-1 [..., c] on the GPU."""
+    shifts = torch.arange(64, device=words.device, dtype=torch.int64)
+    bits = (words.unsqueeze(-1) >> shifts) & 1
+    return (bits.reshape(words.shape[:-1] + (c,)).to(torch.float32) * 2 - 1)
+
+
+def rand_words(gen, *shape):
+    return torch.randint(-2**63, 2**63 - 1, shape, dtype=torch.int64, generator=gen).cuda()
+
+
+@pytest.mark.parametrize("hw,cin,cout,stride", STAGE_SHAPES)
+def test_bconv_batch64_equals_float_convolution(dab, hw, cin, cout, stride):
+    gen = torch.Generator().manual_seed(hw * 1000 + cin + stride)
+    n = 64
+    x = rand_words(gen, n, hw, hw, cin // 64)
+    w = rand_words(gen, cout, 9 * cin // 64)
+    cnt = dab.bconv_3x3(x, w, stride, 1)
+    xs = unpack_pm1(x, cin).permute(0, 3, 1, 2)  # N,C,H,W
+    ws = unpack_pm1(w.reshape(cout, 3, 3, cin // 64), cin).permute(0, 3, 1, 2)
+    torch.backends.cudnn.allow_tf32 = False
+    torch.backends.cuda.matmul.allow_tf32 = False
+    conv = F.conv2d(F.pad(xs, (1, 1, 1, 1), value=-1.0), ws, stride=stride).permute(0, 2, 3, 1)
+    want = (9 * cin - conv) / 2
+    assert torch.equal(cnt, want), (cnt - want).abs().max().item()
+    # batch consistency with the batch-1 launch and a CPU-oracle sample (image 17)
+    one = dab.bconv_3x3(x[17:18].contiguous(), w, stride, 1)
+    assert torch.equal(one[0], cnt[17])
+    xi = x[17].cpu().numpy().view(np.uint64)
+    wi = w.cpu().numpy().view(np.uint64)
+    cpu = orc.baseline_bconv(xi, wi, 3, 3, 1, 1, stride, stride)
+    np.testing.assert_array_equal(cnt[17].cpu().numpy(), cpu)
+
+
+@pytest.mark.parametrize("hw,cin,cout,stride", [(56, 64, 64, 1), (14, 256, 256, 1), (28, 128, 256, 2)])
+def test_bconv_complement_symmetry(dab, hw, cin, cout, stride):
+    gen = torch.Generator().manual_seed(99)
+    x = rand_words(gen, 8, hw, hw, cin // 64)
+    w = rand_words(gen, cout, 9 * cin // 64)
+    a = dab.bconv_3x3(x, w, stride, 1)
+    b = dab.bconv_3x3(~x, w, stride, 1)
+    s = (a + b)
+    interior = s[:, 1:-1, 1:-1] if stride == 1 else s[:, 1:, 1:][:, :-1, :-1]
+    assert (interior == 9 * cin).all()
+
+
+def test_bgemm_config2_linearity_and_float_reference(dab):
+    m, n, k = 512, 3136, 72
+    gen = torch.Generator().manual_seed(5)
+    a = rand_words(gen, k, m)
+    b = rand_words(gen, n, k)
+    c = torch.zeros((n, m), dtype=torch.float32, device="cuda")
+    dab.bgemm(m, n, k, a, m, b, k, c, m)
+    first = c.clone()
+    dab.bgemm(m, n, k, a, m, b, k, c, m)
+    assert torch.equal(c, 2 * first)  # C is accumulated into
+    av = unpack_pm1(a.t().contiguous(), k * 64)  # m, K
+    bv = unpack_pm1(b, k * 64)  # n, K
+    want = (k * 64 - bv @ av.t()) / 2
+    assert torch.equal(first, want)
+
+
+def test_bitpack_config2_roundtrip(dab):
+    gen = torch.Generator().manual_seed(6)
+    x = torch.randn((1, 512, 56, 56), generator=gen).cuda()  # NCHW
+    words = dab.bitpack_nchw(x)
+    assert words.shape == (1, 56, 56, 8)
+    back = unpack_pm1(words, 512)  # NHWC +-1
+    want = torch.where(x > 0, 1.0, -1.0).permute(0, 2, 3, 1)
+    assert torch.equal(back, want)
+    nhwc = x.permute(0, 2, 3, 1).contiguous()
+    assert torch.equal(dab.pack_mat(nhwc), words)
+    # batch 64 of the same shape
+    xb = torch.randn((64, 56, 56, 512), generator=gen).cuda()
+    assert torch.equal(unpack_pm1(dab.pack_mat(xb), 512), torch.where(xb > 0, 1.0, -1.0))
+
+
+def test_fused_im2col_batch64_equals_pack_of_unfold(dab):
+    gen = torch.Generator().manual_seed(7)
+    x = torch.randn((64, 28, 28, 128), generator=gen).cuda()
+    col = dab.fused_binarize_im2col(x, 3, 3, 1, 1, 1, 1)
+    assert col.shape == (64 * 28 * 28, 18)
+    # independent gather: zero-pad, take the 9 taps in (kh, kw) order, sign-pack with pack_mat
+    xp = F.pad(x, (0, 0, 1, 1, 1, 1))
+    taps = [xp[:, a:a + 28, b:b + 28, :] for a in range(3) for b in range(3)]
+    gathered = torch.cat(taps, dim=-1).reshape(-1, 9 * 128).contiguous()
+    assert torch.equal(dab.pack_mat(gathered), col)

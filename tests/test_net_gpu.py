@@ -130,3 +130,26 @@ def test_error_paths(mods, tmp_path):
     with pytest.raises(ValueError):
         n.run(np.zeros((1, 8, 8, 3), dtype=np.float32))
     n.close()
+
+
+def test_graph_replay_equals_eager(mods):
+    """Runs 3+ replay a captured HIP graph; every replay must equal the eager result, also with other GPU work
+    and synchronisations in between and with changing inputs."""
+    import torch
+    df, models, net = mods
+    layers, inits, inputs = models.small_bnn(4, hw=16, width=64)
+    buf = df.write_model(layers, inits, inputs)
+    r = np.random.default_rng(9)
+    xs = [r.standard_normal((2, 16, 16, 3)).astype(np.float32) for _ in range(6)]
+    eager = net.Net(batch=2).read_buf(buf)
+    eager.set_use_graph(False)
+    graphed = net.Net(batch=2).read_buf(buf)
+    for i, x in enumerate(xs):
+        eager.run(x)
+        want = eager.get_blob("logits").copy()
+        graphed.run(x)  # runs 0 and 1 eager, run 2 captures, later runs replay
+        got = graphed.get_blob("logits").copy()
+        np.testing.assert_array_equal(got, want, err_msg="run %d" % i)
+        torch.randn(1 << 16, device="cuda").sum().item()  # unrelated eager work and a sync between replays
+    eager.close()
+    graphed.close()
