@@ -18,6 +18,7 @@ from .ops import (  # noqa: F401
     bitpack_nchw,
     col_row_words,
     fconv,
+    fconv_affine_relu,
     fused_binarize_im2col,
     max_pool,
     pack_mat,

@@ -224,7 +224,12 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             const float4 v = *reinterpret_cast<const float4 *>(src + i * 8 * kStageRow);
             const size_t off = off0 + (size_t)i * 8 * ld;
             float4 *d = reinterpret_cast<float4 *>(out + off);
-            *d = epi(v, d, off);
+            // streaming store: the output is not read again by this kernel, and lines that leave the L2 early do
+            // not have to be written back when the kernel ends
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const float4 r = epi(v, d, off);
+            const f32x4 rv = {r.x, r.y, r.z, r.w};
+            __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(d));
         }
     } else {
         const int magic = (65536 + np - 1) / np;  // c / np for c < 512

@@ -153,17 +153,21 @@ FloatConv::FloatConv(NetCP net, css name, css input, css weight, css output, int
       dilation(dilation_) {}
 
 void FloatConv::forward_impl() const {
-    dab_check(dab_fconv(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
-                        input_mat->c, static_cast<const float *>(weight_mat->data),
-                        bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr, weight_mat->h, weight_mat->w, pad_h,
-                        pad_w, stride_h, stride_w, dilation, dilation, output_mat->c,
-                        static_cast<float *>(output_mat->data), stream()));
+    dab_check(dab_fconv_affine_relu(
+        static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
+        static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
+        fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
+        fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
+        pad_h, pad_w, stride_h, stride_w, dilation, dilation, output_mat->c, static_cast<float *>(output_mat->data),
+        stream()));
 }
 
 std::string FloatConv::to_str() const {
     std::stringstream ss;
     ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->c << ", weight " << weight_mat->n
        << "x" << weight_mat->h << "x" << weight_mat->w;
+    if (fused_a) ss << " + Affine";
+    if (fused_relu) ss << " + Relu";
     return ss.str();
 }
 

@@ -38,6 +38,9 @@ class BinConv : public Layer {
 class FloatConv : public Layer {
    public:
     MatP input_mat, weight_mat, bias_mat, output_mat;
+    // Affine (and Relu) layers that follow on the output blob, applied in the convolution's epilogue when set
+    MatP fused_a, fused_b;
+    bool fused_relu = false;
     const int pad_h, pad_w, stride_h, stride_w, dilation;
     FloatConv(NetCP net, css name, css input, css weight, css bias, css output, int pad_h, int pad_w, int stride_h,
               int stride_w, int dilation);

@@ -280,7 +280,8 @@ void Net::prepare(const void *buf) {
     prepared_ = true;
 }
 
-// BinConv -> Affine (-> Add) on the same blob becomes one pass of the direct kernel.  Blob names and contents after
+// BinConv -> Affine (-> Add) on the same blob becomes one pass of the direct kernel, FloatConv -> Affine (-> Relu) one
+// pass of the float convolution.  Blob names and contents after
 // run() are unchanged: the in-place layers wrote into the BinConv output blob anyway.
 void Net::fuse_binconv_epilogues() {
     std::vector<std::shared_ptr<Layer>> out;
@@ -297,6 +298,21 @@ void Net::fuse_binconv_epilogues() {
                 skip = 2;
             }
             out.push_back(bc);
+            i += skip;
+        } else if (auto fc = std::dynamic_pointer_cast<FloatConv>(layers[i])) {
+            // FloatConv -> Affine (-> Relu), all on the convolution's output blob
+            size_t skip = 0;
+            if (af && af->data_mat == fc->output_mat) {
+                fc->fused_a = af->a_mat;
+                fc->fused_b = af->b_mat;
+                skip = 1;
+            }
+            auto re = i + skip + 1 < layers.size() ? std::dynamic_pointer_cast<Relu>(layers[i + skip + 1]) : nullptr;
+            if (re && re->data_mat == fc->output_mat) {
+                fc->fused_relu = true;
+                ++skip;
+            }
+            out.push_back(fc);
             i += skip;
         } else {
             out.push_back(layers[i]);

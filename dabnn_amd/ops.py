@@ -195,6 +195,26 @@ def fconv(x, weight, bias, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h=1, di
     return out
 
 
+def fconv_affine_relu(x, weight, bias, a, b, relu, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h=1, dil_w=1):
+    """fconv with the Affine (a, b; None for none) and Relu layers that follow it applied in the same pass
+    (dabnn/fconv.h:14-76, dabnn/layers/Affine.cpp:10-23, dabnn/layers/Relu.cpp)."""
+    _need(x, torch.float32, "x")
+    _need(weight, torch.float32, "weight")
+    n, h, w, c = x.shape
+    cout = weight.numel() // (kh * kw * c)
+    for name, t in (("bias", bias), ("a", a), ("b", b)):
+        if t is not None:
+            _need(t, torch.float32, name)
+            if t.numel() != cout:
+                raise capi.DabError(capi.DAB_EINVAL, "fconv_affine_relu: %s does not match the channel count" % name)
+    oh, ow = out_dim(h, pad_h, kh, stride_h, dil_h), out_dim(w, pad_w, kw, stride_w, dil_w)
+    out = _empty((n, max(oh, 0), max(ow, 0), cout), torch.float32, x.device)
+    opt = lambda t: _ptr(t) if t is not None else None
+    check(lib.dab_fconv_affine_relu(_ptr(x), n, h, w, c, _ptr(weight), opt(bias), opt(a), opt(b), int(bool(relu)), kh, kw,
+                                    pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, _ptr(out), _stream()))
+    return out
+
+
 def affine_inplace(x, a, b):
     """affine_inplace (dabnn/layers/Affine.cpp:10-23)."""
     _need(x, torch.float32, "x")

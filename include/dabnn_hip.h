@@ -154,6 +154,16 @@ DAB_API int dab_fconv(const float *x, int n, int h, int w, int c, const float *w
               int pad_h, int pad_w, int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *out,
               dab_stream_t stream);
 
+/*
+ * dab_fconv followed in the same pass by the Affine (a, b; both NULL for none) and Relu (relu != 0) layers that
+ * follow a float convolution in the stem of a network: out = relu(a[c]*(conv + bias[c]) + b[c]), each operation
+ * rounded as the separate layers round it (dabnn/layers/Affine.cpp:10-23, dabnn/layers/Relu.cpp).
+ */
+DAB_API int dab_fconv_affine_relu(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                  const float *a, const float *b, int relu, int kh, int kw, int pad_h, int pad_w,
+                                  int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *out,
+                                  dab_stream_t stream);
+
 /* affine_inplace (dabnn/layers/Affine.cpp:10-23): x[..., ch] = a[ch]*x[..., ch] + b[ch]. */
 DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, const float *b, dab_stream_t stream);
 

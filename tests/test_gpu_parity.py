@@ -273,7 +273,8 @@ RTOL = 1e-4
 @pytest.mark.parametrize("n,h,c,cout,k,pad,stride,dil,bias", [
     (1, 4, 2, 2, 3, 1, 1, 1, False), (1, 8, 2, 2, 5, 2, 2, 1, False), (2, 9, 3, 4, 3, 2, 1, 2, True),
     (1, 32, 3, 64, 7, 3, 2, 1, False), (2, 7, 64, 128, 1, 0, 1, 1, False), (3, 1, 512, 1000, 1, 0, 1, 1, True),
-    (1, 17, 5, 70, 3, 1, 2, 1, True),
+    (1, 17, 5, 70, 3, 1, 2, 1, True), (2, 9, 3, 32, 3, 1, 2, 1, False), (1, 23, 16, 20, 3, 1, 1, 1, True),
+    (1, 12, 7, 200, 5, 2, 1, 1, True), (130, 1, 33, 65, 1, 0, 1, 1, False), (1, 40, 8, 8, 3, 1, 1, 1, False),
 ])
 def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
     r = rng(40)
@@ -285,6 +286,31 @@ def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
     want = np.stack([orc.fconv(img, wgt, bv, k, k, pad, pad, stride, stride, dil, dil) for img in x])
     scale = np.abs(want).max()
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+
+
+@pytest.mark.parametrize("affine,relu,bias", [(True, True, False), (True, False, True), (False, True, True)])
+def test_fconv_affine_relu_equals_separate_layers(dab, affine, relu, bias):
+    """One pass gives what FpConv2D, Affine and Relu give one after the other, bit for bit against the separate GPU
+    layers and within the float tolerance against the CPU restatement."""
+    r = rng(43)
+    n, h, c, cout, k = 2, 19, 3, 32, 3
+    x = r.standard_normal((n, h, h, c)).astype(np.float32)
+    wgt = r.standard_normal((cout, k, k, c)).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32) if bias else None
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    got = dab.fconv_affine_relu(dev_f(x), dev_f(wgt), dev_f(bv) if bias else None, dev_f(a) if affine else None,
+                                dev_f(b) if affine else None, relu, k, k, 1, 1, 2, 2).cpu().numpy()
+    sep = dab.fconv(dev_f(x), dev_f(wgt), dev_f(bv) if bias else None, k, k, 1, 1, 2, 2)
+    if affine:
+        dab.affine_inplace(sep, dev_f(a), dev_f(b))
+    sep = sep.cpu().numpy()
+    want = np.stack([orc.fconv(img, wgt, bv, k, k, 1, 1, 2, 2) for img in x])
+    if affine:
+        want = np.stack([orc.affine_inplace(img.copy(), a, b) for img in want])
+    if relu:
+        sep, want = np.maximum(sep, 0), np.maximum(want, 0)
+    np.testing.assert_array_equal(got, sep)
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * np.abs(want).max())
 
 
 def test_fconv_ramp_cases_of_reference_tests(dab):
