@@ -11,12 +11,19 @@ namespace dab {
 // depth = kh*kw*c in the reference's (kh, kw, c) order (dabnn/fconv.h:33-41,
 // dabnn/im2col.h:14-47).  This is the one GEMM-shaped fp32 layer of the path, so
 // it runs on the matrix cores: v_mfma_f32_32x32x2_f32, fp32 in and fp32 accumulate.
-// A 256-thread block owns a 128 x BN output tile (BN = 32, 64 or 128) as four
-// wave tiles; 16-deep slices of the gathered image patch and of the weights are
-// staged in two LDS buffers, the next slice fetched into registers while the
-// current one is multiplied.  A depth index is the same for all lanes of a wave
-// while it loads, so its decoding into (tap row, tap column, channel) runs once
-// per wave on the scalar unit.
+//
+// A 256-thread block owns a BM x BN output tile.  SK-deep slices of the gathered
+// image patch and of the weights are staged in two LDS buffers, rows = pixel /
+// output channel, depth contiguous; the next slice is fetched into registers
+// while the current one is multiplied.  Lanes of a load run along the depth,
+// which is contiguous in memory for both operands (channels, then the taps of a
+// kernel row), so a wave touches a few cache lines per load.
+// The four waves split the tile (KSPLIT = 1) or, for problems too small to give
+// every CU a big tile, all work on one 32 x 32 tile and split each slice's depth
+// (KSPLIT = 4); their partial sums are then added in a fixed order through LDS.
+// Which depth index sits in which of the instruction's two depth slots does not
+// matter as long as both operands agree: a lane takes four consecutive depths
+// with one 16-byte LDS read and uses them in four instructions.
 // Epilogue: + bias, then optionally the Affine (a*v + b, two roundings) and Relu
 // layers that follow the convolution, in the reference's order of operations.
 struct FconvArgs {
@@ -38,67 +45,91 @@ struct FconvArgs {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kFM = 128, kFK = 16;
+// Addressing: all three tensors are reached through buffer descriptors that start at the block's own first image /
+// weight row / output row, so 32-bit byte offsets suffice for tensors of any size, reads past the end of the
+// descriptor (rows beyond the last pixel or channel) return zero and such writes are dropped.  An element that is
+// padding, or whose depth index is past K, gets the offset kOob, which is out of range for every descriptor.
+constexpr uint32_t kOob = 0x80000000u;     // descriptors here are shorter than 2^30 bytes
+constexpr uint32_t kOobRow = 0x40000000u;  // kOobRow + kOob and kOobRow + (anything < 2^30) stay out of range
 
-template <int BN>
+template <int BM, int BN, int SK, int KSPLIT, bool PADDED>
 __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
-    constexpr int WAVES_N = BN >= 64 ? 2 : 1, WAVES_M = 4 / WAVES_N;
-    constexpr int WTM = kFM / WAVES_M, WTN = BN / WAVES_N;  // wave tile
-    constexpr int TM = WTM / 32, TN = WTN / 32;             // 32 x 32 matrix-core tiles per wave
-    constexpr int BPT = BN / 16;                            // weights fetched per thread and slice
-    // row strides of 32 (mod 64) floats: the two half-waves of a fragment read land in different banks
-    constexpr int AS = kFM + 32, BS = (BN % 64 == 32) ? BN : BN + 32;
-    __shared__ float As[2][kFK][AS];  // [k][pixel]
-    __shared__ float Bs[2][kFK][BS];  // [k][cout]
+    constexpr int WAVES_MN = 4 / KSPLIT;
+    constexpr int WAVES_N = (WAVES_MN >= 2 && BN >= 64) ? 2 : 1, WAVES_M = WAVES_MN / WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;  // wave tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;            // 32 x 32 matrix-core tiles per wave
+    constexpr int RP = 256 / SK;                           // tile rows fetched per pass of the block
+    constexpr int APT = BM / RP, BPT = BN / RP;            // loads per thread and slice
+    constexpr int RS = SK + 4;                             // LDS row stride: 16-byte reads of 16 lanes hit 64 banks once
+    static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
+    static_assert(SK == 16 * KSPLIT && APT >= 1 && BPT >= 1, "slice");
+    __shared__ __attribute__((aligned(16))) float As[2][BM][RS];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN][RS];
+    __shared__ float red[KSPLIT > 1 ? KSPLIT * 16 * 64 : 1];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    const int m0 = blockIdx.x * kFM, n0 = blockIdx.y * BN;
+    const int ks = wave / WAVES_MN, wm = (wave % WAVES_MN) / WAVES_N, wn = wave % WAVES_N;
+    const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
 
-    // A loader: this thread always fetches pixel (tid % 128), depth rows (tid / 128) + 2*i
-    const int l_m = tid & 127, l_kk = __builtin_amdgcn_readfirstlane(tid >> 7);
-    const int pix = m0 + l_m;
-    const bool pix_ok = pix < p.M;
-    int y0 = 0, x0 = 0;
-    const float *xpix = p.x;
-    if (pix_ok) {
-        const uint32_t t = p.div_ow.div((uint32_t)pix);
-        const int ox = pix - t * p.ow;
-        const uint32_t img = p.div_oh.div(t);
-        const int oy = t - img * p.oh;
-        y0 = oy * p.stride_h - p.pad_h, x0 = ox * p.stride_w - p.pad_w;
-        // signed 64-bit arithmetic: y0 and x0 are negative inside the padding; the pointer is only used in bounds
-        xpix = p.x + (((long long)img * p.h + y0) * p.wd + x0) * p.c;
+    // descriptors relative to this block's first image, first weight row and first output row
+    const int img0 = (int)p.div_oh.div(p.div_ow.div((uint32_t)m0));
+    const int img_elems = p.h * p.wd * p.c;
+    const long long x_left = (long long)(p.n - img0) * img_elems * 4;
+    const auto x_rsrc = make_rsrc(p.x + (size_t)img0 * img_elems, (uint32_t)(x_left < kOobRow ? x_left : kOobRow));
+    const int rows_n = p.cout - n0 < BN ? p.cout - n0 : BN, rows_m = p.M - m0 < BM ? p.M - m0 : BM;
+    const auto w_rsrc = make_rsrc(p.w + (size_t)n0 * p.K, (uint32_t)rows_n * p.K * 4u);
+    const auto o_rsrc = make_rsrc(p.out + (size_t)m0 * p.cout, (uint32_t)rows_m * p.cout * 4u);
+
+    // loader: depth l_k of the slice, tile rows l_r + RP*i
+    const int l_k = tid % SK, l_r = tid / SK;
+    uint32_t a_base[APT];  // byte offset of (image, y0, x0, channel 0) from the descriptor's start, modulo 2^32
+    int a_y0[PADDED ? APT : 1], a_x0[PADDED ? APT : 1];
+#pragma unroll
+    for (int i = 0; i < APT; ++i) {
+        const int pix = m0 + l_r + RP * i;
+        if (pix < p.M) {
+            const uint32_t t = p.div_ow.div((uint32_t)pix);
+            const int ox = pix - (int)t * p.ow;
+            const int img = (int)p.div_oh.div(t);
+            const int oy = (int)t - img * p.oh;
+            const int y0 = oy * p.stride_h - p.pad_h, x0 = ox * p.stride_w - p.pad_w;
+            a_base[i] = (uint32_t)((((img - img0) * p.h + y0) * p.wd + x0) * p.c) * 4u;
+            if (PADDED) a_y0[i] = y0, a_x0[i] = x0;
+        } else {
+            a_base[i] = kOobRow;
+            if (PADDED) a_y0[i] = -(1 << 30), a_x0[i] = 0;  // every tap fails the bounds test
+        }
     }
-    // B loader: depth (tid % 16), output channels (tid / 16) + 16*j
-    const int b_k = tid & 15, b_n = tid >> 4;
+    uint32_t b_row[BPT];
+#pragma unroll
+    for (int j = 0; j < BPT; ++j) b_row[j] = (uint32_t)(l_r + RP * j) * p.K * 4u;
 
-    float a_reg[8], b_reg[BPT];
+    float a_reg[APT], b_reg[BPT];
     auto fetch = [&](int k0) {
+        const int k = k0 + l_k;
+        const bool k_ok = k < p.K;
+        const int tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
+        const int ty = (int)p.div_kw.div((uint32_t)tap), tx = tap - ty * p.kw;
+        const int dy = ty * p.dil_h, dx = tx * p.dil_w;
+        const uint32_t delta = k_ok ? (uint32_t)((dy * p.wd + dx) * p.c + ch) * 4u : kOob;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int k = k0 + l_kk + 2 * i;
-            float v = 0.f;
-            if (k < p.K) {
-                const int tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
-                const int ty = (int)p.div_kw.div((uint32_t)tap), tx = tap - ty * p.kw;
-                const int dy = ty * p.dil_h, dx = tx * p.dil_w;
-                const int y = y0 + dy, xx = x0 + dx;
-                if (pix_ok && (unsigned)y < (unsigned)p.h && (unsigned)xx < (unsigned)p.wd)
-                    v = xpix[(dy * p.wd + dx) * p.c + ch];
+        for (int i = 0; i < APT; ++i) {
+            uint32_t off = a_base[i] + delta;
+            if (PADDED) {
+                const int y = a_y0[i] + dy, xx = a_x0[i] + dx;
+                off = ((unsigned)y < (unsigned)p.h && (unsigned)xx < (unsigned)p.wd) ? off : kOob;
             }
-            a_reg[i] = v;
+            a_reg[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)off, 0, 0));
         }
+        const uint32_t k4 = k_ok ? (uint32_t)k * 4u : kOob;
 #pragma unroll
-        for (int j = 0; j < BPT; ++j) {
-            const int co = n0 + b_n + 16 * j, k = k0 + b_k;
-            b_reg[j] = (co < p.cout && k < p.K) ? p.w[(size_t)co * p.K + k] : 0.f;
-        }
+        for (int j = 0; j < BPT; ++j)
+            b_reg[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, (int)(b_row[j] + k4), 0, 0));
     };
     auto commit = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) As[buf][l_kk + 2 * i][l_m] = a_reg[i];
+        for (int i = 0; i < APT; ++i) As[buf][l_r + RP * i][l_k] = a_reg[i];
 #pragma unroll
-        for (int j = 0; j < BPT; ++j) Bs[buf][b_k][b_n + 16 * j] = b_reg[j];
+        for (int j = 0; j < BPT; ++j) Bs[buf][l_r + RP * j][l_k] = b_reg[j];
     };
 
     f32x16 acc[TM][TN];
@@ -109,57 +140,83 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    // fragment addressing of v_mfma_f32_32x32x2_f32: lane l supplies row/column l % 32 at depth l / 32
+    // operand lane l of the instruction: row / column l % 32, depth slot l / 32
     const int f_k = lane >> 5, f_i = lane & 31;
     fetch(0);
     commit(0);
     __syncthreads();
     int buf = 0;
-    for (int k0 = 0; k0 < p.K; k0 += kFK, buf ^= 1) {
-        const bool more = k0 + kFK < p.K;
-        if (more) fetch(k0 + kFK);
+    for (int k0 = 0; k0 < p.K; k0 += SK, buf ^= 1) {
+        const bool more = k0 + SK < p.K;
+        if (more) fetch(k0 + SK);
 #pragma unroll
-        for (int kp = 0; kp < kFK / 2; ++kp) {
-            float a[TM], b[TN];
+        for (int g = 0; g < 2; ++g) {  // this wave's 16 depths of the slice, 8 at a time
+            const int kb = ks * 16 + g * 8 + f_k * 4;
+            float4 a4[TM], b4[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) a[i] = As[buf][kp * 2 + f_k][wm * WTM + i * 32 + f_i];
+            for (int i = 0; i < TM; ++i) a4[i] = *reinterpret_cast<const float4 *>(&As[buf][wm * WTM + i * 32 + f_i][kb]);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) b[j] = Bs[buf][kp * 2 + f_k][wn * WTN + j * 32 + f_i];
+            for (int j = 0; j < TN; ++j) b4[j] = *reinterpret_cast<const float4 *>(&Bs[buf][wn * WTN + j * 32 + f_i][kb]);
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < TN; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i].x, b4[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i].y, b4[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i].z, b4[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4[i].w, b4[j].w, acc[i][j], 0, 0, 0);
+                }
         }
         // the other buffer was last read before the barrier that ended the previous slice
         if (more) commit(buf ^ 1);
         __syncthreads();
     }
 
-    // accumulator element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l % 32
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const int co = n0 + wn * WTN + j * 32 + f_i;
-        if (co >= p.cout) continue;
-        const float bias = p.bias ? p.bias[co] : 0.f;
-        const float fa = p.aff_a ? p.aff_a[co] : 0.f, fb = p.aff_a ? p.aff_b[co] : 0.f;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int m = m0 + wm * WTM + i * 32 + 8 * (e / 4) + 4 * f_k + (e % 4);
-                if (m >= p.M) continue;
-                {
+    // row: tile row of the output element; rows past the last pixel are past the end of the output descriptor
+    auto emit = [&](int row, uint32_t co_off, float v, float bias, float fa, float fb) {
 #pragma clang fp contract(off)
-                    float v = acc[i][j][e];
-                    if (p.bias) v = v + bias;
-                    if (p.aff_a) {
-                        const float prod = fa * v;
-                        v = prod + fb;
-                    }
-                    if (p.relu) v = v > 0.f ? v : 0.f;
-                    p.out[(size_t)m * p.cout + co] = v;
-                }
-            }
+        if (p.bias) v = v + bias;
+        if (p.aff_a) {
+            const float prod = fa * v;
+            v = prod + fb;
+        }
+        if (p.relu) v = v > 0.f ? v : 0.f;
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), o_rsrc,
+                                              (int)((uint32_t)row * p.cout * 4u + co_off), 0, 0);
+    };
+
+    // accumulator element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l % 32
+    if (KSPLIT == 1) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int co = n0 + wn * WTN + j * 32 + f_i;
+            const bool co_ok = co < p.cout;
+            const float bias = (p.bias && co_ok) ? p.bias[co] : 0.f;
+            const float fa = (p.aff_a && co_ok) ? p.aff_a[co] : 0.f, fb = (p.aff_a && co_ok) ? p.aff_b[co] : 0.f;
+            const uint32_t co_off = co_ok ? (uint32_t)co * 4u : kOob;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    emit(wm * WTM + i * 32 + 8 * (e / 4) + 4 * f_k + (e % 4), co_off, acc[i][j][e], bias, fa, fb);
+        }
+    } else {
+        // one 32 x 32 tile: the waves' partial sums are added in wave order, four accumulator elements per thread
+#pragma unroll
+        for (int e = 0; e < 16; ++e) red[(ks * 16 + e) * 64 + lane] = acc[0][0][e];
+        __syncthreads();
+        const int co = n0 + f_i;
+        const bool co_ok = co < p.cout;
+        const float bias = (p.bias && co_ok) ? p.bias[co] : 0.f;
+        const float fa = (p.aff_a && co_ok) ? p.aff_a[co] : 0.f, fb = (p.aff_a && co_ok) ? p.aff_b[co] : 0.f;
+        const uint32_t co_off = co_ok ? (uint32_t)co * 4u : kOob;
+#pragma unroll
+        for (int q = 0; q < 16 / KSPLIT; ++q) {
+            const int e = wave * (16 / KSPLIT) + q;
+            float v = red[e * 64 + lane];
+#pragma unroll
+            for (int s = 1; s < KSPLIT; ++s) v = __fadd_rn(v, red[(s * 16 + e) * 64 + lane]);
+            emit(8 * (e / 4) + 4 * f_k + (e % 4), co_off, v, bias, fa, fb);
         }
     }
 }
@@ -313,21 +370,42 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
     a.cout = cout;
     a.K = kh * kw * c;
     const long long M = (long long)n * a.oh * a.ow;
-    if (M >= (1ll << 31) - kFM || (long long)n * h * w * c >= (1ll << 31))
+    if (M >= (1ll << 31) - 128 || (long long)n * h * w * c >= (1ll << 31))
         return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
     a.M = (int)M;
     a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
     a.kw = kw, a.dil_h = dil_h, a.dil_w = dil_w;
     a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv((uint32_t)kw);
     hipStream_t s = as_stream(stream);
-    const unsigned gx = (unsigned)((M + kFM - 1) / kFM);
-    if (cout <= 32) {
-        hipLaunchKernelGGL(fconv_kernel<32>, dim3(gx, 1), dim3(256), 0, s, a);
-    } else if (cout <= 64) {
-        hipLaunchKernelGGL(fconv_kernel<64>, dim3(gx, 1), dim3(256), 0, s, a);
+    // byte offsets inside a block's descriptors stay below 2^30: the images its 128 pixels come from, 128 weight
+    // rows, 128 output rows
+    const long long span_imgs = 128 / ((long long)a.oh * a.ow) + 2;
+    if (span_imgs * h * w * c * 4 >= (1ll << 30) || 128ll * a.K * 4 >= (1ll << 30) || 128ll * cout * 4 >= (1ll << 30))
+        return fail(DAB_EUNSUPPORTED, "%s: image, filter or channel count too large for 32-bit tile offsets", fn);
+    // without padding every tap of every window is inside the image and the bounds test is dropped
+    const bool padded = pad_h != 0 || pad_w != 0 || (a.oh - 1) * stride_h + (kh - 1) * dil_h >= h ||
+                        (a.ow - 1) * stride_w + (kw - 1) * dil_w >= w;
+    const int bn = cout <= 32 ? 32 : cout <= 64 ? 64 : 128;
+    const long long big_tiles = ((M + 127) / 128) * ((cout + bn - 1) / bn);
+#define DAB_FCONV_LAUNCH(BM, BN, SK, KSPLIT)                                                             \
+    do {                                                                                                 \
+        const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN));                \
+        if (padded)                                                                                      \
+            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, true>), grid, dim3(256), 0, s, a);      \
+        else                                                                                             \
+            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false>), grid, dim3(256), 0, s, a);     \
+    } while (0)
+    if (big_tiles < simd_count() / 4) {
+        // fewer big tiles than CUs: 32 x 32 tiles, each slice's depth split over the block's waves
+        DAB_FCONV_LAUNCH(32, 32, 64, 4);
+    } else if (bn == 32) {
+        DAB_FCONV_LAUNCH(128, 32, 16, 1);
+    } else if (bn == 64) {
+        DAB_FCONV_LAUNCH(128, 64, 16, 1);
     } else {
-        hipLaunchKernelGGL(fconv_kernel<128>, dim3(gx, (unsigned)((cout + 127) / 128)), dim3(256), 0, s, a);
+        DAB_FCONV_LAUNCH(128, 128, 16, 1);
     }
+#undef DAB_FCONV_LAUNCH
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }

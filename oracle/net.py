@@ -12,53 +12,101 @@ import numpy as np
 import oracle as orc
 
 
-def run_model(layers, initializers, x, record=None):
-    """x: float32 [H, W, C].  record: optional dict that receives a copy of each BinConv's raw counts."""
-    blobs = {t["name"]: t for t in initializers}
-    act = {"data": np.ascontiguousarray(x, dtype=np.float32)}
-
+def _apply(layer, act, blobs, record=None):
+    """Runs one layer on the activations in ``act`` (in-place layers alias their output name to the input array)."""
     def weights(name):
         t = blobs[name]
         return np.asarray(t["data"]), t["shape"]
 
-    for layer in layers:
-        ty = layer["type"]
-        if ty in ("FpConv2D", "BinConv2D"):
-            src = act[layer["input"]]
-            w, shape = weights(layer["weight"])
-            cout, kh, kw, cin = shape
-            pad_h, pad_w = layer["pads"][0], layer["pads"][1]
-            sh, sw = layer["strides"][0], layer["strides"][1]
-            if ty == "BinConv2D":
-                wp = w.reshape(cout, -1)
-                if cin == 64 and (kh, kw) != (3, 3):
-                    out = orc.baseline_bconv(orc.pack_mat(src), wp, kh, kw, pad_h, pad_w, sh, sw)
-                else:
-                    out, _ = orc.binconv_forward(src, wp, kh, kw, pad_h, pad_w, sh, sw)
-                if record is not None:
-                    record[layer["output"]] = out.copy()
+    ty = layer["type"]
+    if ty in ("FpConv2D", "BinConv2D"):
+        src = act[layer["input"]]
+        w, shape = weights(layer["weight"])
+        cout, kh, kw, cin = shape
+        pad_h, pad_w = layer["pads"][0], layer["pads"][1]
+        sh, sw = layer["strides"][0], layer["strides"][1]
+        if ty == "BinConv2D":
+            wp = w.reshape(cout, -1)
+            if cin == 64 and (kh, kw) != (3, 3):
+                out = orc.baseline_bconv(orc.pack_mat(src), wp, kh, kw, pad_h, pad_w, sh, sw)
             else:
-                bias = np.asarray(blobs[layer["bias"]]["data"]) if layer.get("bias") else None
-                out = orc.fconv(src, w.reshape(cout, kh, kw, cin), bias, kh, kw, pad_h, pad_w, sh, sw)
-            act[layer["output"]] = out
-        elif ty == "Affine":
-            buf = act[layer["input"]]
-            orc.affine_inplace(buf, np.asarray(blobs[layer["a"]]["data"]), np.asarray(blobs[layer["b"]]["data"]))
-            act[layer["output"]] = buf
-        elif ty == "Add":
-            buf = act[layer["input1"]]
-            orc.add_inplace(buf, act[layer["input2"]])
-            act[layer["output"]] = buf
-        elif ty == "Relu":
-            buf = act[layer["input"]]
-            np.maximum(buf, 0, out=buf)
-            act[layer["output"]] = buf
-        elif ty in ("MaxPool", "AvePool"):
-            src = act[layer["input"]]
-            kh, kw = layer["kernel_shape"]
-            fn = orc.max_pool if ty == "MaxPool" else orc.ave_pool
-            act[layer["output"]] = fn(src, kh, kw, layer["pads"][0], layer["pads"][1], layer["strides"][0],
-                                      layer["strides"][1])
+                out, _ = orc.binconv_forward(src, wp, kh, kw, pad_h, pad_w, sh, sw)
+            if record is not None:
+                record[layer["output"]] = out.copy()
         else:
-            raise RuntimeError("Not supported op " + ty)
+            bias = np.asarray(blobs[layer["bias"]]["data"]) if layer.get("bias") else None
+            out = orc.fconv(src, w.reshape(cout, kh, kw, cin), bias, kh, kw, pad_h, pad_w, sh, sw)
+        act[layer["output"]] = out
+    elif ty == "Affine":
+        buf = act[layer["input"]]
+        orc.affine_inplace(buf, np.asarray(blobs[layer["a"]]["data"]), np.asarray(blobs[layer["b"]]["data"]))
+        act[layer["output"]] = buf
+    elif ty == "Add":
+        buf = act[layer["input1"]]
+        orc.add_inplace(buf, act[layer["input2"]])
+        act[layer["output"]] = buf
+    elif ty == "Relu":
+        buf = act[layer["input"]]
+        np.maximum(buf, 0, out=buf)
+        act[layer["output"]] = buf
+    elif ty in ("MaxPool", "AvePool"):
+        src = act[layer["input"]]
+        kh, kw = layer["kernel_shape"]
+        fn = orc.max_pool if ty == "MaxPool" else orc.ave_pool
+        act[layer["output"]] = fn(src, kh, kw, layer["pads"][0], layer["pads"][1], layer["strides"][0],
+                                  layer["strides"][1])
+    else:
+        raise RuntimeError("Not supported op " + ty)
+
+
+def run_model(layers, initializers, x, record=None):
+    """x: float32 [H, W, C].  record: optional dict that receives a copy of each BinConv's raw counts."""
+    blobs = {t["name"]: t for t in initializers}
+    act = {"data": np.ascontiguousarray(x, dtype=np.float32)}
+    for layer in layers:
+        _apply(layer, act, blobs, record)
     return act
+
+
+_INPLACE = {"Affine": "input", "Add": "input1", "Relu": "input"}
+
+
+def run_segments(layers, initializers, fetch):
+    """Layer-by-layer check with the other implementation's own activations as inputs.
+
+    A sign network amplifies a one-ulp difference in a float layer into flipped bits downstream, so two correct
+    implementations drift apart end to end.  Here the layers are cut into segments (a layer that writes a new blob
+    plus the in-place layers that later rewrite that blob); every segment is evaluated on the CPU from ``fetch(name)`` -- the
+    final content of the input blobs as the implementation under test holds them after its run -- and yields
+    (output blob name, type of the first layer, CPU result).  Valid when a blob is only read after the in-place layers
+    on it have run, which holds for the graphs the converter emits (tools/onnx2bnn/OnnxConverter.cpp:583-639).
+    """
+    blobs = {t["name"]: t for t in initializers}
+    root = {}
+
+    def r(name):
+        while name in root:
+            name = root[name]
+        return name
+
+    segs, owner = [], {}
+    for layer in layers:
+        key = _INPLACE.get(layer["type"])
+        if key is not None and r(layer[key]) in owner:
+            owner[r(layer[key])].append(layer)  # joins the segment of the blob it rewrites, wherever that started
+        else:
+            segs.append([layer])
+            owner[r(layer[key]) if key is not None else layer["output"]] = segs[-1]
+        if key is not None:
+            root[layer["output"]] = layer[key]
+    for seg in segs:
+        act = {}
+        first = seg[0]
+        for key in ("input", "input1", "input2"):
+            if key in first:
+                act[first[key]] = np.array(fetch(r(first[key])), dtype=np.float32, copy=True)
+        for layer in seg:
+            if layer is not first and layer["type"] == "Add":
+                act[layer["input2"]] = np.array(fetch(r(layer["input2"])), dtype=np.float32, copy=True)
+            _apply(layer, act, blobs)
+        yield r(seg[-1]["output"]), first["type"], act[seg[-1]["output"]]

@@ -26,6 +26,26 @@ def close(got, want):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
 
 
+def check_every_segment(n, layers, inits, image):
+    """Every layer group of the device run against the CPU restatement fed with the device's own input blobs:
+    bit-exact after a binary convolution (counts are integers; Affine and Add round alike on both sides) and for
+    max pooling, 1e-4 relative after float convolutions and average pooling."""
+    checked = 0
+    for name, first_type, want in orc_net.run_segments(layers, inits, lambda b: n.get_blob(b)[image]):
+        got = n.get_blob(name)[image]
+        if first_type in ("BinConv2D", "MaxPool", "Affine", "Add", "Relu"):
+            np.testing.assert_array_equal(got, want, err_msg=name)
+        else:
+            close(got, want)
+        checked += 1
+    return checked
+
+
+def drift_ok(got, want):
+    """End to end only a loose bound holds: one flipped sign early on moves the logits by about a percent."""
+    assert np.corrcoef(got.ravel(), want.ravel())[0, 1] > 0.98
+
+
 def test_small_net_matches_cpu_layer_loop(mods):
     df, models, net = mods
     layers, inits, inputs = models.small_bnn(1, hw=16, width=64)
@@ -38,9 +58,9 @@ def test_small_net_matches_cpu_layer_loop(mods):
     n.run(x)
     logits = n.get_blob("logits").reshape(batch, -1)
     for i in range(batch):
-        rec = {}
-        cpu = orc_net.run_model(layers, inits, x[i], record=rec)
-        close(logits[i], cpu["logits"].ravel())
+        assert check_every_segment(n, layers, inits, i) == 7
+        cpu = orc_net.run_model(layers, inits, x[i])
+        drift_ok(logits[i], cpu["logits"])
         # packed input of every BinConv: bit-exact unless a float sits within rounding of zero
         for blk in ("b0", "b1", "b2"):
             packed = n.get_blob("binaized_for_%s_cnt_cal" % blk)[i]
@@ -102,9 +122,9 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     logits = n.get_blob("logits").reshape(2, -1)
     assert logits.shape == (2, 1000)
     for i in range(2):
-        cpu = orc_net.run_model(layers, inits, x[i])
-        close(logits[i], cpu["logits"].ravel())
-        close(n.get_blob("pool1_out")[i], cpu["pool1_out"])
+        assert check_every_segment(n, layers, inits, i) >= 20
+    cpu = orc_net.run_model(layers, inits, x[0])
+    drift_ok(logits[0], cpu["logits"])
     n.set_profile(True)
     n.run(x)
     report = n.time_report()

@@ -366,3 +366,21 @@ def test_pools_vs_torch(h, w, c, k, pad, stride):
     mx = F.max_pool2d(xt, k, stride, pad)[0].permute(1, 2, 0).numpy()
     np.testing.assert_allclose(orc.ave_pool(x, k, k, pad, pad, stride, stride), avg, rtol=1e-5, atol=1e-6)
     np.testing.assert_array_equal(orc.max_pool(x, k, k, pad, pad, stride, stride), mx)
+
+
+def test_run_segments_fed_with_its_own_blobs_reproduces_the_layer_loop():
+    """The segment-wise evaluation used to check a device run layer by layer, given the CPU run's own final blobs,
+    must return exactly those blobs: in-place layers join the segment of the blob they rewrite, also when other
+    layers (the shortcut of a down-sampling block) sit in between."""
+    from dabnn_amd import models
+    from oracle import net as orc_net
+    for layers, inits, hw in (models.small_bnn(1, hw=16, width=64) [:2] + (16,), models.bireal18(3, stem=True)[:2] + (64,)):
+        x = np.random.default_rng(5).standard_normal((hw, hw, 3)).astype(np.float32)
+        if hw == 64:  # Bi-Real-18 graph on a 64 x 64 image: the 7 x 7 pool before the classifier becomes 2 x 2
+            layers = [dict(l, kernel_shape=[2, 2]) if l["name"] == "pool5" else l for l in layers]
+        cpu = orc_net.run_model(layers, inits, x)
+        count = 0
+        for name, _, want in orc_net.run_segments(layers, inits, lambda b: cpu[b]):
+            np.testing.assert_array_equal(want, cpu[name])
+            count += 1
+        assert count == (7 if hw == 16 else 28)
