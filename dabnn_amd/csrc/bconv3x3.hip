@@ -47,14 +47,23 @@ struct ItemUnits {
     static constexpr int value = Q >= 4 ? 1 : 4 / Q;
 };
 
-// The second launch bound asks the register allocator for 3 resident waves per SIMD at 512 channels
-// (144 of the 512/3 = 168 available VGPRs hold the activations), 4 otherwise (the staging buffers allow no more).
+// Resident waves per SIMD the kernel is built for, and the staging window that lets them fit the CU's LDS:
+// the activations take 18*CW VGPRs, so 64 and 128 channels leave room for 8 and 6 waves (with the 16-channel
+// window, 5 KB per wave), 256 channels for 4 and 512 channels (144 of 512/3 = 168 VGPRs) for 3.
+template <int CW>
+struct Residency {
+    static constexpr int waves_per_simd = CW == 1 ? 8 : CW == 2 ? 6 : CW == 4 ? 4 : 3;
+    static constexpr int window = CW <= 2 ? 16 : 32;
+};
+
 template <int CW, bool FUSED>
-__global__ __launch_bounds__(64 * kWavesPerBlock, CW == 8 ? 3 : 4) void bconv3x3_kernel(const BconvArgs p) {
+__global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
     constexpr int Q = UnitChannels<CW>::value;
     constexpr int S = ItemUnits<Q>::value;
-    constexpr int WU = 32 / Q;  // units per 32-channel staging window
+    constexpr int WCH = Residency<CW>::window;
+    constexpr int WU = WCH / Q;  // units per staging window
+    constexpr int kStageBytes = Stage<WCH>::bytes;
     __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -112,17 +121,17 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, CW == 8 ? 3 : 4) void bconv3x3
         for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
         unit_rowmajor<K32, Q, (CW >= 2 ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
         const int slot = cg % WU;
-        stage_put<Q>(stage, lane, slot * Q, acc);
+        stage_put<WCH, Q>(stage, lane, slot * Q, acc);
 
         const bool last_in_tile = cg == p.n_groups - 1;
         if (slot == WU - 1 || last_in_tile || u == u1 - 1) {
             if constexpr (FUSED) {
                 EpiAffineAdd epi;
                 epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
-                stage_flush(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
+                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
                             epi);
             } else {
-                stage_flush(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
+                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
                             EpiStore());
             }
             ch_lo = 0;

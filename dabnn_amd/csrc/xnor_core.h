@@ -154,20 +154,26 @@ __device__ __forceinline__ void unit_colmajor(const void *wbase, uint32_t stride
 }
 
 // ---------------------------------------------------------------- output staging
-// A wave parks up to 32 channels (4 units) of its 64 pixels in LDS, one row
-// per pixel, and writes them out transposed: 8 consecutive lanes cover the
-// 128 contiguous bytes of one pixel, so every store instruction writes whole
-// cache lines instead of 64 scattered 16-byte pieces.
-constexpr int kStageRow = 144;                // 32 channels * 4 B + 16 B pad: conflict-free b128 access
-constexpr int kStageBytes = 64 * kStageRow;   // per wave
+// A wave parks a window of WCH channels (32 or 16) of its 64 pixels in LDS, one
+// row per pixel, and writes them out transposed: WCH/4 consecutive lanes cover
+// the WCH*4 contiguous bytes of one pixel, so every store instruction writes
+// whole or half cache lines instead of 64 scattered 16-byte pieces.  The narrow
+// window halves the LDS a wave holds, which is what bounds the resident waves
+// of the kernels with few activation registers.
+template <int WCH>
+struct Stage {
+    static constexpr int row = WCH * 4 + 16;  // + 16 B pad: conflict-free 16-byte writes of one lane per row
+    static constexpr int bytes = 64 * row;    // per wave
+    static constexpr int parts = WCH / 4;     // 16-byte parts per pixel row
+};
 
 // Parks the Q results of a lane at channel offset ch_off (multiple of Q) of its row.
-template <int Q>
+template <int WCH, int Q>
 __device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch_off, const uint32_t (&acc)[Q]) {
     float f[Q];
 #pragma unroll
     for (int q = 0; q < Q; ++q) f[q] = __uint_as_float(acc[q]) - kAccBias;
-    unsigned char *row = stage + lane * kStageRow + ch_off * 4;
+    unsigned char *row = stage + lane * Stage<WCH>::row + ch_off * 4;
     if constexpr (Q == 2) {
         *reinterpret_cast<float2 *>(row) = make_float2(f[0], f[1]);
     } else {
@@ -207,22 +213,23 @@ struct EpiAffineAdd {
 };
 
 // Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
-// 32-channel window that starts at channel cbase.  out is [pixel][ld] floats;
+// WCH-channel window that starts at channel cbase.  out is [pixel][ld] floats;
 // pixels >= total are skipped.
-template <class Epi>
+template <int WCH, class Epi>
 __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
                                             int tile, int total, int cbase, int p_lo, int p_hi, Epi epi) {
     __builtin_amdgcn_wave_barrier();
     const int np = p_hi - p_lo + 1;  // 16-byte parts per pixel row
-    if (np == 8 && (tile + 1) * 64 <= total) {
-        const int pr0 = lane >> 3, part = lane & 7;
-        const unsigned char *src = stage + pr0 * kStageRow + part * 16;
+    constexpr int NP = Stage<WCH>::parts, ROW = Stage<WCH>::row, PPI = 64 / NP;  // PPI pixels per store instruction
+    if (np == NP && (tile + 1) * 64 <= total) {
+        const int pr0 = lane / NP, part = lane % NP;
+        const unsigned char *src = stage + pr0 * ROW + part * 16;
         const size_t off0 = ((size_t)tile * 64 + pr0) * ld + cbase + part * 4;
         epi.prepare(cbase + part * 4);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float4 v = *reinterpret_cast<const float4 *>(src + i * 8 * kStageRow);
-            const size_t off = off0 + (size_t)i * 8 * ld;
+        for (int i = 0; i < NP; ++i) {
+            const float4 v = *reinterpret_cast<const float4 *>(src + i * PPI * ROW);
+            const size_t off = off0 + (size_t)i * PPI * ld;
             float4 *d = reinterpret_cast<float4 *>(out + off);
             // streaming store: the output is not read again by this kernel, and lines that leave the L2 early do
             // not have to be written back when the kernel ends
@@ -239,7 +246,7 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             const int part = p_lo + (c - pr * np);
             const int pix = tile * 64 + pr;
             if (pix < total) {
-                const float4 v = *reinterpret_cast<const float4 *>(stage + pr * kStageRow + part * 16);
+                const float4 v = *reinterpret_cast<const float4 *>(stage + pr * ROW + part * 16);
                 const size_t off = (size_t)pix * ld + cbase + part * 4;
                 float4 *d = reinterpret_cast<float4 *>(out + off);
                 epi.prepare(cbase + part * 4);
@@ -270,7 +277,10 @@ inline int resident_blocks_per_cu(Kernel kernel, int block_threads) {
 
 inline int pick_wave_count(int n_items, int blocks_per_cu, int waves_per_block) {
     long long w = (long long)(simd_count() / 4) * blocks_per_cu * waves_per_block;
-    if (w > n_items) w = n_items;
+    // Fewer items than resident waves: one item per wave.  When that still fills more than half of the machine,
+    // two items per wave are faster, because a wave fetches its lane-resident operand once for both; smaller
+    // problems are latency-bound and keep one item per wave.
+    if (w >= n_items) w = 2ll * n_items > w ? (n_items + 1) / 2 : n_items;
     if (w < 1) w = 1;
     return (int)((w + waves_per_block - 1) / waves_per_block * waves_per_block);
 }
