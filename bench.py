@@ -29,6 +29,11 @@ STAGE_SHAPES = [  # (H=W, Cin, Cout, stride)
     (56, 64, 128, 2), (28, 128, 256, 2), (14, 256, 512, 2),
 ]
 BATCH = 64
+# HBM traffic of the headline workload per kernel launch (bytes, mean of the seven shapes), measured with
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --profile-mode` (summary: profiles/bconv3x3_config3_b64.md),
+# next to the algorithmic bytes (packed input + weights + fp32 output).
+TRAFFIC_BYTES_PER_LAUNCH = 27.38e6
+ALGORITHMIC_BYTES_PER_LAUNCH = 21.10e6
 
 
 def out_dim(size, pad, k, stride):
@@ -111,9 +116,11 @@ def main():
         torch.cuda.synchronize()
         pgraph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(pgraph):
+            for _ in range(args.steps):
+                step()
+        for _ in range(args.warmup):
             step()
-        for _ in range(args.warmup + args.steps):
-            pgraph.replay()
+        pgraph.replay()
         torch.cuda.synchronize()
         print(json.dumps({"profile_mode": True, "steps": args.steps, "warmup": args.warmup,
                           "shapes": ["%dx%d %d->%d s%d b%d" % (hw, hw, ci, co, st, BATCH) for (hw, ci, co, st) in STAGE_SHAPES]}))
@@ -121,16 +128,18 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # The K timed steps are one HIP graph (7*K kernel nodes, launched once): a graph launch costs the GPU about
+    # 10 us before its first kernel starts, which a caller that runs layer after layer pays once per network pass,
+    # not once per layer group.
     step_graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(step_graph):
-        step()
-    step_graph.replay()
+        for _ in range(args.steps):
+            step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(args.steps):
-        step_graph.replay()
+    step_graph.replay()
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -145,7 +154,7 @@ def main():
         dur_sum += d
         per_shape.append({"shape": "%dx%d %d->%d s%d b%d" % (hw, hw, cin, cout, stride, BATCH), "us": round(d * 1e6, 2),
                           "Tbinop/s": round(ops / d / 1e12, 1), "frac": round(ops / d / peak_binops, 3)})
-    # launch-level roofline figure: all seven launches of the timed region (events around the graph replays)
+    # launch-level roofline figure: all 7*K launches of the timed region (events around the graph launch)
     step_seconds = e0.elapsed_time(e1) * 1e-3 / args.steps
     achieved = step_binops / step_seconds
 
@@ -294,11 +303,14 @@ def main():
                    "batch": BATCH, "binops_per_step": step_binops, "device": torch.cuda.get_device_name(0),
                    "cus": cus, "clock_mhz": khz / 1e3},
         "roofline": {"bound": "valu_popcount", "achieved": achieved / 1e12, "peak": peak_binops / 1e12,
-                     "unit": "Tbinop/s", "frac": achieved / peak_binops, "traffic": None,
+                     "unit": "Tbinop/s", "frac": achieved / peak_binops, "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic_algorithmic": ALGORITHMIC_BYTES_PER_LAUNCH,
                      "kernel": "bconv3x3_kernel", "note": "peak = CUs*64 lanes*clock*32 binop (one v_xor_b32 + one "
                      "v_bcnt_u32_b32 per 32 bits); achieved = binops of the seven launches of a step / their HIP-event time "
-                     "in the timed region (average launch = 1/7 of that); per-shape figures under workloads are each "
-                     "shape launched back to back, with warm caches"},
+                     "in the timed region (all K steps are one HIP graph; average launch = 1/7 of a step); traffic = HBM "
+                     "bytes per launch averaged over the seven shapes from rocprofv3 FETCH_SIZE and WRITE_SIZE runs of "
+                     "--profile-mode, each scaled by the same counter's reading for a 256 MiB copy (x2.0 and x1.0); "
+                     "per-shape figures under workloads are each shape launched back to back"},
         "cpu_baseline": cpu,
         "workloads": workloads,
     }

@@ -116,6 +116,19 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
             }
         }
 
+        // The SIMD issues from its oldest wave first, so with equal priorities the waves of a SIMD finish one after
+        // the other and the last one runs alone at the single-wave issue rate.  Priority by remaining work keeps
+        // them level: they reach their last units together.
+        const int left = CW >= 4 ? u1 - u - 1 : 0;  // measured: no gain with 7-8 resident waves per SIMD
+        if (left >= 3) {
+            __builtin_amdgcn_s_setprio(3);
+        } else if (left == 2) {
+            __builtin_amdgcn_s_setprio(2);
+        } else if (left == 1) {
+            __builtin_amdgcn_s_setprio(1);
+        } else {
+            __builtin_amdgcn_s_setprio(0);
+        }
         uint32_t acc[Q];
 #pragma unroll
         for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
