@@ -4,14 +4,15 @@
 // (zeros where a tap falls outside the image) zero-extended to a multiple of
 // 128 and sign-packed; row_words = ceil(kh*kw*c/128)*2 words.
 //
-// A wave produces one output word per compare: lane l looks at element
-// 64*wi + l of the row and the lane mask of (value > 0) is the word.  When c
-// is a multiple of 64 a word never straddles two taps, so the 64 lanes read
-// 256 contiguous bytes of one tap.  The general path resolves tap and channel
-// per lane.
-// HBM-bound on paper (each input float is needed kh*kw times but comes from
-// L2 after the first touch): 4 bytes per input element read, 8 bytes per
-// output word written.
+// A wave produces one word per compare: lane l looks at 64 consecutive
+// floats and the lane mask of (value > 0) is the word.  When c is a multiple
+// of 64 a word never straddles two taps, so binarising and gathering commute:
+// a block packs the input rows that its output rows touch into LDS once
+// (every float is read about once, not kh*kw times) and then writes its col
+// rows by copying words out of LDS.  The general path resolves tap and
+// channel per lane for every output word.
+// HBM-bound: 4 bytes per input element read (plus the halo rows shared by
+// neighbouring blocks), 8 bytes per output word written.
 #include "common.h"
 
 namespace dab {
@@ -26,11 +27,66 @@ struct Im2colArgs {
     int len;  // kh*kw*c
     long long n_words;
     FastDiv div_row_words, div_ow, div_oh, div_c, div_kw, div_cw;
+    int rows_per_block, blocks_per_image;  // tiled kernel only
 };
 
 constexpr int kIm2colWavesPerBlock = 4;
 
-// c % 64 == 0.  Lane l first decodes output word g0 + l of the chunk (row ->
+// c % 64 == 0, one block per (image, run of rows_per_block output rows).  Phase 1 packs the input rows
+// [y_lo, y_hi) that the run's windows reach (contiguous in memory) into LDS, one 256-byte load and one compare per
+// word; phase 2 writes the run's col rows, which are contiguous too, one word per lane from LDS or zero.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void fused_binarize_im2col_tiled_kernel(const Im2colArgs p) {
+    extern __shared__ uint64_t packed[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int img = blockIdx.x / p.blocks_per_image, rb = blockIdx.x - img * p.blocks_per_image;
+    const int cw = p.c >> 6;
+    const int oy0 = rb * p.rows_per_block;
+    const int oy1 = oy0 + p.rows_per_block < p.oh ? oy0 + p.rows_per_block : p.oh;
+    int y_lo = oy0 * p.stride_h - p.pad_h;
+    int y_hi = (oy1 - 1) * p.stride_h - p.pad_h + (p.kh - 1) * p.dil_h + 1;
+    y_lo = y_lo < 0 ? 0 : y_lo;
+    y_hi = y_hi > p.h ? p.h : y_hi;
+    const int n_in = y_hi > y_lo ? (y_hi - y_lo) * p.w * cw : 0;  // words to pack
+    const float *src = p.x + ((size_t)img * p.h + y_lo) * p.w * p.c;
+    for (int j0 = wib * 64; j0 < n_in; j0 += THREADS) {
+        const int cnt = n_in - j0 < 64 ? n_in - j0 : 64;
+        uint64_t mine = 0;
+        // always 64 independent loads in flight; the words past the end repeat the last one and are not stored
+        float v[64];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) v[i] = src[(size_t)(j0 + (i < cnt ? i : cnt - 1)) * 64 + lane];
+#pragma unroll
+        for (int i = 0; i < 64; ++i) {
+            const uint64_t word = __ballot(v[i] > 0.0f);
+            mine = (lane == i) ? word : mine;
+        }
+        if (lane < cnt) packed[j0 + lane] = mine;
+    }
+    __syncthreads();
+    const int n_out = (oy1 - oy0) * p.ow * p.row_words;
+    uint64_t *dst = p.col + ((size_t)img * p.oh + oy0) * p.ow * p.row_words;
+    const int n_taps = p.kh * p.kw;
+    for (int g = tid; g < n_out; g += THREADS) {
+        const uint32_t pix = p.div_row_words.div((uint32_t)g);
+        const int wi = g - pix * p.row_words;
+        const uint32_t oyl = p.div_ow.div(pix);
+        const int ox = pix - oyl * p.ow;
+        const uint32_t tap = p.div_cw.div((uint32_t)wi);  // >= kh*kw for the zero padding word
+        const int k = wi - tap * cw;
+        const uint32_t a = p.div_kw.div(tap);
+        const int b = tap - a * p.kw;
+        const int y = (oy0 + (int)oyl) * p.stride_h - p.pad_h + (int)a * p.dil_h;
+        const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
+        // a row inside the image is inside [y_lo, y_hi): the run's windows span exactly that range
+        const bool ok = (int)tap < n_taps && y >= 0 && y < p.h && xx >= 0 && xx < p.w;
+        dst[g] = ok ? packed[((y - y_lo) * p.w + xx) * cw + k] : 0ull;
+    }
+}
+
+// c % 64 == 0, for images whose rows do not fit the tiled kernel's LDS budget.
+// Lane l first decodes output word g0 + l of the chunk (row ->
 // image/oy/ox, word -> tap/channel word, bounds test) with ordinary vector
 // arithmetic, 64 words at once; the 64 element offsets are then broadcast one
 // by one (v_readlane) and every word becomes one coalesced 256-byte load, one
@@ -141,10 +197,27 @@ extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, in
     a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
     a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv((uint32_t)kw);
     a.div_cw = FastDiv((uint32_t)(c >= 64 ? c / 64 : 1));
+    a.rows_per_block = 0, a.blocks_per_image = 0;
     const long long chunks = (a.n_words + 63) / 64;
     long long blocks = (chunks + kIm2colWavesPerBlock - 1) / kIm2colWavesPerBlock;
     const long long cap = (long long)simd_count() * 8;
     if (blocks > cap) blocks = cap;
+    if (c % 64 == 0) {
+        // rows per block: as many as fit 48 KB of packed input rows, fewer while that leaves CUs without a block
+        // (measured best: about one 512-thread block per CU; more rows per block re-read fewer halo rows)
+        const int cw = c / 64;
+        auto lds_bytes = [&](int r) { return ((long long)(r - 1) * stride_h + (long long)(kh - 1) * dil_h + 1) * w * cw * 8; };
+        int r = a.oh;
+        while (r > 1 && (lds_bytes(r) > 48 * 1024 || (long long)n * ((a.oh + r - 1) / r) < simd_count() / 4)) r = (r + 1) / 2;
+        if (lds_bytes(r) <= 48 * 1024) {
+            a.rows_per_block = r;
+            a.blocks_per_image = (a.oh + r - 1) / r;
+            hipLaunchKernelGGL(fused_binarize_im2col_tiled_kernel<512>, dim3((unsigned)(n * a.blocks_per_image)), dim3(512),
+                               (size_t)lds_bytes(r), as_stream(stream), a);
+            DAB_LAUNCH_CHECK();
+            return DAB_OK;
+        }
+    }
     if (c % 64 == 0)
         hipLaunchKernelGGL(fused_binarize_im2col_aligned_kernel, dim3((unsigned)blocks), dim3(64 * kIm2colWavesPerBlock), 0,
                            as_stream(stream), a);

@@ -89,6 +89,9 @@ def test_pad_bit(dab, n, h, w, cw, ph, pw):
     (1, 8, 8, 128, 3, 1, 1, 1), (2, 8, 8, 64, 3, 1, 2, 1), (1, 7, 9, 192, 3, 1, 1, 1), (1, 6, 6, 128, 5, 2, 2, 1),
     (2, 5, 5, 3, 3, 1, 1, 1), (1, 4, 4, 100, 1, 0, 1, 1), (1, 10, 10, 64, 3, 2, 1, 2), (1, 28, 28, 128, 3, 1, 1, 1),
     (1, 14, 14, 256, 3, 1, 2, 1), (2, 7, 7, 512, 3, 1, 1, 1), (1, 3, 3, 128, 3, 0, 2, 1),
+    # enough images that a block of the row-tiled kernel takes several output rows (2, 8 = whole image, 2 with a
+    # ragged last block, 1 under stride 2)
+    (40, 14, 14, 64, 3, 1, 1, 1), (300, 8, 8, 64, 3, 1, 1, 1), (150, 9, 9, 64, 5, 2, 2, 2), (70, 12, 10, 128, 3, 1, 2, 1),
 ])
 def test_fused_binarize_im2col(dab, n, h, w, c, k, pad, stride, dil):
     x = special_floats((n, h, w, c), 4)
