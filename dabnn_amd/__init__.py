@@ -14,6 +14,7 @@ from .ops import (  # noqa: F401
     ave_pool,
     bconv_3x3,
     bconv_3x3_affine_add,
+    bconv_3x3_affine_add_sign,
     bgemm,
     bitpack_nchw,
     col_row_words,

@@ -26,10 +26,11 @@ struct BconvArgs {
     int items_per_wave, items_extra;  // split of the work items over the waves
     uint32_t x_bytes;
     FastDiv div_ow, div_oh, div_groups;
-    // fused epilogue (FUSED kernels only): out = a*cnt + b (+ shortcut)
+    // fused epilogue (MODE >= 1 kernels only): out = a*cnt + b (+ shortcut); MODE 2 also writes sign bits of out
     const float *epi_a;
     const float *epi_b;
     const float *epi_shortcut;
+    unsigned char *epi_bits;
 };
 
 constexpr int kWavesPerBlock = 4;
@@ -41,11 +42,16 @@ struct UnitChannels {
 };
 
 // Work items handed to waves are runs of S units so that a wave's share of a
-// pixel row always starts and ends on a 16-byte boundary (4 channels).
-template <int Q>
+// pixel row always starts and ends on a 16-byte boundary (4 channels) -- on
+// 8 channels when the epilogue also writes sign bits, one whole byte of them.
+template <int Q, bool EMIT>
 struct ItemUnits {
-    static constexpr int value = Q >= 4 ? 1 : 4 / Q;
+    static constexpr int align = EMIT ? 8 : 4;
+    static constexpr int value = Q >= align ? 1 : align / Q;
 };
+
+// MODE 0: raw counts.  1: + Affine (+ Add).  2: the same and a sign-packed copy of the result.
+constexpr int kModeCounts = 0, kModeAffineAdd = 1, kModeAffineAddSign = 2;
 
 // Resident waves per SIMD the kernel is built for, and the staging window that lets them fit the CU's LDS:
 // the activations take 18*CW VGPRs, so 64 and 128 channels leave room for 8 and 6 waves (with the 16-channel
@@ -56,11 +62,11 @@ struct Residency {
     static constexpr int window = CW <= 2 ? 16 : 32;
 };
 
-template <int CW, bool FUSED>
+template <int CW, int MODE>
 __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
     constexpr int Q = UnitChannels<CW>::value;
-    constexpr int S = ItemUnits<Q>::value;
+    constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     constexpr int WCH = Residency<CW>::window;
     constexpr int WU = WCH / Q;  // units per staging window
     constexpr int kStageBytes = Stage<WCH>::bytes;
@@ -138,14 +144,20 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
 
         const bool last_in_tile = cg == p.n_groups - 1;
         if (slot == WU - 1 || last_in_tile || u == u1 - 1) {
-            if constexpr (FUSED) {
+            if constexpr (MODE == kModeAffineAddSign) {
+                EpiAffineAddSign epi;
+                epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+                epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
+                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
+                                 (slot * Q + Q - 1) >> 2, epi);
+            } else if constexpr (MODE == kModeAffineAdd) {
                 EpiAffineAdd epi;
                 epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
-                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
-                            epi);
+                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
+                                 (slot * Q + Q - 1) >> 2, epi);
             } else {
-                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2, (slot * Q + Q - 1) >> 2,
-                            EpiStore());
+                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
+                                 (slot * Q + Q - 1) >> 2, EpiStore());
             }
             ch_lo = 0;
         }
@@ -159,19 +171,19 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
     }
 }
 
-template <int CW, bool FUSED>
+template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW>::value;
-    constexpr int S = ItemUnits<Q>::value;
+    constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, FUSED>, 64 * kWavesPerBlock);
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE>, 64 * kWavesPerBlock);
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
     a.div_groups = FastDiv((uint32_t)a.n_groups);
-    hipLaunchKernelGGL((bconv3x3_kernel<CW, FUSED>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
+    hipLaunchKernelGGL((bconv3x3_kernel<CW, MODE>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }
@@ -179,8 +191,8 @@ static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
 }  // namespace dab
 
 static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
-                         int stride, int pad, const float *a_coef, const float *b_coef, const float *shortcut, bool fused,
-                         float *out, dab_stream_t stream) {
+                         int stride, int pad, const float *a_coef, const float *b_coef, const float *shortcut, int mode,
+                         float *out, uint64_t *out_packed, dab_stream_t stream) {
     using namespace dab;
     DAB_REQUIRE(x && wgt && out, "%s: null pointer", fn);
     DAB_REQUIRE(n > 0 && h > 0 && w > 0 && cin > 0 && cout > 0, "%s: non-positive dimension", fn);
@@ -192,6 +204,12 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     DAB_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wgt) & 7) == 0 &&
                     (reinterpret_cast<uintptr_t>(out) & 15) == 0,
                 "%s: buffers must be 16-byte aligned", fn);
+    const bool fused = mode != kModeCounts;
+    if (mode == kModeAffineAddSign) {
+        DAB_REQUIRE(out_packed, "%s: null pointer", fn);
+        DAB_REQUIRE((reinterpret_cast<uintptr_t>(out_packed) & 7) == 0, "%s: buffers must be 16-byte aligned", fn);
+        if (cout % 64 != 0) return fail(DAB_EUNSUPPORTED, "%s: cout %d is not a multiple of 64", fn, cout);
+    }
     if (fused) {
         DAB_REQUIRE(a_coef && b_coef, "%s: null affine coefficients", fn);
         DAB_REQUIRE((reinterpret_cast<uintptr_t>(a_coef) & 15) == 0 && (reinterpret_cast<uintptr_t>(b_coef) & 15) == 0 &&
@@ -202,6 +220,7 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     BconvArgs a;
     a.x = x, a.w = wgt, a.out = out;
     a.epi_a = a_coef, a.epi_b = b_coef, a.epi_shortcut = shortcut;
+    a.epi_bits = reinterpret_cast<unsigned char *>(out_packed);
     a.H = h, a.W = w;
     a.OH = out_dim(h, pad, 3, 1, stride), a.OW = out_dim(w, pad, 3, 1, stride);
     const long long total = (long long)n * a.OH * a.OW;
@@ -214,31 +233,39 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     a.div_ow = FastDiv((uint32_t)a.OW), a.div_oh = FastDiv((uint32_t)a.OH);
     const long long tiles = (total + 63) / 64;
     hipStream_t s = as_stream(stream);
-    if (fused) {
-        switch (cin) {
-            case 64: return launch_bconv3x3<1, true>(a, tiles, s);
-            case 128: return launch_bconv3x3<2, true>(a, tiles, s);
-            case 256: return launch_bconv3x3<4, true>(a, tiles, s);
-            default: return launch_bconv3x3<8, true>(a, tiles, s);
-        }
+    switch (mode * 16 + cin / 64) {
+        case kModeCounts * 16 + 1: return launch_bconv3x3<1, kModeCounts>(a, tiles, s);
+        case kModeCounts * 16 + 2: return launch_bconv3x3<2, kModeCounts>(a, tiles, s);
+        case kModeCounts * 16 + 4: return launch_bconv3x3<4, kModeCounts>(a, tiles, s);
+        case kModeCounts * 16 + 8: return launch_bconv3x3<8, kModeCounts>(a, tiles, s);
+        case kModeAffineAdd * 16 + 1: return launch_bconv3x3<1, kModeAffineAdd>(a, tiles, s);
+        case kModeAffineAdd * 16 + 2: return launch_bconv3x3<2, kModeAffineAdd>(a, tiles, s);
+        case kModeAffineAdd * 16 + 4: return launch_bconv3x3<4, kModeAffineAdd>(a, tiles, s);
+        case kModeAffineAdd * 16 + 8: return launch_bconv3x3<8, kModeAffineAdd>(a, tiles, s);
+        case kModeAffineAddSign * 16 + 1: return launch_bconv3x3<1, kModeAffineAddSign>(a, tiles, s);
+        case kModeAffineAddSign * 16 + 2: return launch_bconv3x3<2, kModeAffineAddSign>(a, tiles, s);
+        case kModeAffineAddSign * 16 + 4: return launch_bconv3x3<4, kModeAffineAddSign>(a, tiles, s);
+        case kModeAffineAddSign * 16 + 8: return launch_bconv3x3<8, kModeAffineAddSign>(a, tiles, s);
     }
-    switch (cin) {
-        case 64: return launch_bconv3x3<1, false>(a, tiles, s);
-        case 128: return launch_bconv3x3<2, false>(a, tiles, s);
-        case 256: return launch_bconv3x3<4, false>(a, tiles, s);
-        default: return launch_bconv3x3<8, false>(a, tiles, s);
-    }
+    return fail(DAB_EINVAL, "%s: bad mode", fn);
 }
 
 extern "C" int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
                             int pad, float *out, dab_stream_t stream) {
-    return bconv3x3_impl("dab_bconv3x3", x, n, h, w, cin, wgt, cout, stride, pad, nullptr, nullptr, nullptr, false, out,
-                         stream);
+    return bconv3x3_impl("dab_bconv3x3", x, n, h, w, cin, wgt, cout, stride, pad, nullptr, nullptr, nullptr, dab::kModeCounts,
+                         out, nullptr, stream);
 }
 
 extern "C" int dab_bconv3x3_affine_add(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
                                        int stride, int pad, const float *a, const float *b, const float *shortcut,
                                        float *out, dab_stream_t stream) {
-    return bconv3x3_impl("dab_bconv3x3_affine_add", x, n, h, w, cin, wgt, cout, stride, pad, a, b, shortcut, true, out,
-                         stream);
+    return bconv3x3_impl("dab_bconv3x3_affine_add", x, n, h, w, cin, wgt, cout, stride, pad, a, b, shortcut,
+                         dab::kModeAffineAdd, out, nullptr, stream);
+}
+
+extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
+                                            int stride, int pad, const float *a, const float *b, const float *shortcut,
+                                            float *out, uint64_t *out_packed, dab_stream_t stream) {
+    return bconv3x3_impl("dab_bconv3x3_affine_add_sign", x, n, h, w, cin, wgt, cout, stride, pad, a, b, shortcut,
+                         dab::kModeAffineAddSign, out, out_packed, stream);
 }

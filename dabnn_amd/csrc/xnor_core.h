@@ -183,14 +183,19 @@ __device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch
 }
 
 // What happens to four consecutive channels of one pixel on their way out.
-//   EpiStore      out = cnt                                  (the reference's BinConv output)
-//   EpiAffineAdd  out = a[ch]*cnt + b[ch] (+ shortcut)       (BinConv -> Affine -> Add of a residual block in one
-//                 pass; multiply, add and add are rounded separately, exactly like the three layers)
+//   EpiStore          out = cnt                                  (the reference's BinConv output)
+//   EpiAffineAdd      out = a[ch]*cnt + b[ch] (+ shortcut)       (BinConv -> Affine -> Add of a residual block in one
+//                     pass; multiply, add and add are rounded separately, exactly like the three layers)
+//   EpiAffineAddSign  the same, and bit (out > 0) of every result goes to a packed copy of the output, the words the
+//                     next binary convolution would otherwise make by reading the fp32 blob again
+//                     (pack_mat, dabnn/bitpack.h:277-293)
 struct EpiStore {
+    static constexpr bool kEmit = false;
     __device__ __forceinline__ void prepare(int) {}
     __device__ __forceinline__ float4 operator()(float4 v, const float4 *, size_t) const { return v; }
 };
 struct EpiAffineAdd {
+    static constexpr bool kEmit = false;
     const float *a;
     const float *b;
     const float *shortcut;  // may be null; same layout as out
@@ -211,6 +216,20 @@ struct EpiAffineAdd {
         return r;
     }
 };
+struct EpiAffineAddSign : EpiAffineAdd {
+    static constexpr bool kEmit = true;
+    unsigned char *bits;  // packed output, [pixel][bits_ld] bytes, bit c%8 of byte c/8 = (out[pixel][c] > 0)
+    int bits_ld;          // cout / 8
+};
+
+__device__ __forceinline__ uint32_t sign_nibble(float4 r) {
+    return (uint32_t)(r.x > 0.0f) | ((uint32_t)(r.y > 0.0f) << 1) | ((uint32_t)(r.z > 0.0f) << 2) | ((uint32_t)(r.w > 0.0f) << 3);
+}
+// v | (v of lane + N within the row of 16 lanes; zero past the row's end): DPP row_shl:N
+template <int N>
+__device__ __forceinline__ uint32_t or_from_lane_above(uint32_t v) {
+    return v | (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x100 + N, 0xF, 0xF, true);
+}
 
 // Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
 // WCH-channel window that starts at channel cbase.  out is [pixel][ld] floats;
@@ -237,6 +256,20 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             const float4 r = epi(v, d, off);
             const f32x4 rv = {r.x, r.y, r.z, r.w};
             __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(d));
+            if constexpr (Epi::kEmit) {
+                // the NP lanes of a pixel hold its window's sign bits, four each: gather them in the first lane
+                uint32_t w = sign_nibble(r) << (4 * part);
+                w = or_from_lane_above<1>(w);
+                w = or_from_lane_above<2>(w);
+                if constexpr (NP == 8) w = or_from_lane_above<4>(w);
+                unsigned char *bd = epi.bits + ((size_t)tile * 64 + pr0 + i * PPI) * epi.bits_ld + (cbase >> 3);
+                if (part == 0) {
+                    if constexpr (NP == 8)
+                        *reinterpret_cast<uint32_t *>(bd) = w;
+                    else
+                        *reinterpret_cast<uint16_t *>(bd) = (uint16_t)w;
+                }
+            }
         }
     } else {
         const int magic = (65536 + np - 1) / np;  // c / np for c < 512
@@ -245,12 +278,22 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             const int pr = (c * magic) >> 16;
             const int part = p_lo + (c - pr * np);
             const int pix = tile * 64 + pr;
+            uint32_t nib = 0;
             if (pix < total) {
                 const float4 v = *reinterpret_cast<const float4 *>(stage + pr * ROW + part * 16);
                 const size_t off = (size_t)pix * ld + cbase + part * 4;
                 float4 *d = reinterpret_cast<float4 *>(out + off);
                 epi.prepare(cbase + part * 4);
-                *d = epi(v, d, off);
+                const float4 r = epi(v, d, off);
+                *d = r;
+                if constexpr (Epi::kEmit) nib = sign_nibble(r);
+            }
+            if constexpr (Epi::kEmit) {
+                // p_lo and np are even here (a wave's share of a pixel row is whole bytes of sign bits), so the two
+                // halves of a byte sit in lanes 2k and 2k+1
+                uint32_t w = nib << (4 * (part & 1));
+                w = or_from_lane_above<1>(w);
+                if (pix < total && !(part & 1)) epi.bits[(size_t)pix * epi.bits_ld + ((cbase + part * 4) >> 3)] = (unsigned char)w;
             }
         }
     }

@@ -88,8 +88,14 @@ void BinConv::forward_impl() const {
         case DIRECT_CONV: {
             // pack_mat + (pad +) bconv_3x3, dabnn/layers/BinConv.cpp:146-150
             auto *packed = static_cast<uint64_t *>(binarized_mat->data);
-            dab_check(dab_bitpack_nhwc(x, packed, (int64_t)n * h * w, c, s));
-            if (fused_a) {
+            if (!input_prepacked) dab_check(dab_bitpack_nhwc(x, packed, (int64_t)n * h * w, c, s));
+            if (fused_a && fused_sign_out) {
+                dab_check(dab_bconv3x3_affine_add_sign(
+                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n, stride_h, pad_h,
+                    static_cast<const float *>(fused_a->data), static_cast<const float *>(fused_b->data),
+                    fused_shortcut ? static_cast<const float *>(fused_shortcut->data) : nullptr, out,
+                    static_cast<uint64_t *>(fused_sign_out->data), s));
+            } else if (fused_a) {
                 dab_check(dab_bconv3x3_affine_add(
                     packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n, stride_h, pad_h,
                     static_cast<const float *>(fused_a->data), static_cast<const float *>(fused_b->data),
@@ -122,7 +128,9 @@ std::string BinConv::to_str() const {
     ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->elem_c << ", weight "
        << weight_mat->n << "x" << kernel_h() << "x" << kernel_w() << ", pad " << pad_h << "," << pad_w << ", stride "
        << stride_h << "," << stride_w << ", method " << (method() == DIRECT_CONV ? "DIRECT_CONV" : "BGEMM");
+    if (input_prepacked) ss << ", packed input from the previous block";
     if (fused_a) ss << (fused_shortcut ? " + Affine + Add" : " + Affine");
+    if (fused_sign_out) ss << " + Sign";
     return ss.str();
 }
 

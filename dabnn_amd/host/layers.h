@@ -23,6 +23,11 @@ class BinConv : public Layer {
     // Set by Net::prepare when the layers that follow are Affine (and Add) on this layer's output and the direct
     // kernel applies: the three run as one pass with identical results.
     MatP fused_a, fused_b, fused_shortcut;
+    // Also set by Net::prepare: the fused pass of this layer writes the sign-packed copy of its result that the next
+    // direct BinConv on that blob needs (fused_sign_out = that layer's binarized_mat), and a layer whose packed input
+    // is made that way skips its own pack_mat (input_prepacked).
+    MatP fused_sign_out;
+    bool input_prepacked = false;
 
     BinConv(NetCP net, css name, css input, css weight, css output, int pad_h, int pad_w, int stride_h, int stride_w);
     void forward_impl() const override;

@@ -1,5 +1,7 @@
 #include "net.h"
 
+#include <algorithm>
+
 #include <hip/hip_runtime_api.h>
 
 #include <fstream>
@@ -280,10 +282,68 @@ void Net::prepare(const void *buf) {
     prepared_ = true;
 }
 
-// BinConv -> Affine (-> Add) on the same blob becomes one pass of the direct kernel, FloatConv -> Affine (-> Relu) one
-// pass of the float convolution.  Blob names and contents after
-// run() are unchanged: the in-place layers wrote into the BinConv output blob anyway.
+// Blobs a layer reads and writes (in-place layers do both).
+static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &reads, std::vector<const Mat *> &writes) {
+    reads.clear(), writes.clear();
+    if (auto bc = std::dynamic_pointer_cast<BinConv>(l)) {
+        reads = {bc->input_mat.get()};
+        writes = {bc->output_mat.get(), bc->binarized_mat.get(), bc->col_mat.get()};
+    } else if (auto fc = std::dynamic_pointer_cast<FloatConv>(l)) {
+        reads = {fc->input_mat.get()};
+        writes = {fc->output_mat.get()};
+    } else if (auto af = std::dynamic_pointer_cast<Affine>(l)) {
+        reads = writes = {af->data_mat.get()};
+    } else if (auto ad = std::dynamic_pointer_cast<Add>(l)) {
+        reads = {ad->input1_mat.get(), ad->input2_mat.get()};
+        writes = {ad->input1_mat.get()};
+    } else if (auto re = std::dynamic_pointer_cast<Relu>(l)) {
+        reads = writes = {re->data_mat.get()};
+    } else if (auto ap = std::dynamic_pointer_cast<AvePool>(l)) {
+        reads = {ap->input_mat.get()};
+        writes = {ap->output_mat.get()};
+    } else if (auto mp = std::dynamic_pointer_cast<MaxPool>(l)) {
+        reads = {mp->input_mat.get()};
+        writes = {mp->output_mat.get()};
+    }
+}
+
+static bool contains(const std::vector<const Mat *> &v, const Mat *m) {
+    for (const Mat *x : v)
+        if (x == m) return true;
+    return false;
+}
+
+// Three rewrites of the layer list; blob names and contents after run() are unchanged, because the in-place layers
+// wrote into the convolution's output blob anyway.
+//  1. In a down-sampling block the converter emits BinConv, Affine, [AvePool, FpConv2D, Affine], Add: the shortcut
+//     branch in brackets neither reads nor writes the BinConv's blobs, so BinConv and Affine move behind it, next to
+//     their Add.
+//  2. BinConv -> Affine (-> Add) on the same blob becomes one pass of the direct kernel, FloatConv -> Affine (-> Relu)
+//     one pass of the float convolution.
+//  3. When the blob such a fused BinConv completes is the input of a later direct BinConv, the pass also writes that
+//     layer's packed input and the later layer skips its pack_mat.
 void Net::fuse_binconv_epilogues() {
+    std::vector<const Mat *> rd, wr;
+    for (size_t i = 0; i + 2 < layers.size(); ++i) {
+        auto bc = std::dynamic_pointer_cast<BinConv>(layers[i]);
+        auto af = std::dynamic_pointer_cast<Affine>(layers[i + 1]);
+        if (!bc || !af || af->data_mat != bc->output_mat) continue;
+        size_t j = i + 2;
+        bool movable = true;
+        for (; j < layers.size(); ++j) {
+            layer_io(layers[j], rd, wr);
+            if (contains(rd, bc->output_mat.get()) || contains(wr, bc->output_mat.get())) break;
+            // the branch must not disturb what the BinConv reads, nor use its scratch
+            if (contains(wr, bc->input_mat.get()) || contains(rd, bc->binarized_mat.get()) ||
+                contains(wr, bc->binarized_mat.get()) || rd.empty())
+                movable = false;
+        }
+        auto ad = j < layers.size() ? std::dynamic_pointer_cast<Add>(layers[j]) : nullptr;
+        if (!movable || j == i + 2 || !ad || ad->input1_mat != bc->output_mat || ad->input2_mat == bc->output_mat) continue;
+        std::rotate(layers.begin() + i, layers.begin() + i + 2, layers.begin() + j);  // [bc, af, branch...] -> [branch..., bc, af]
+        i = j;  // continue behind the Add
+    }
+
     std::vector<std::shared_ptr<Layer>> out;
     for (size_t i = 0; i < layers.size(); ++i) {
         auto bc = std::dynamic_pointer_cast<BinConv>(layers[i]);
@@ -319,6 +379,23 @@ void Net::fuse_binconv_epilogues() {
         }
     }
     layers.swap(out);
+
+    for (size_t i = 0; i < layers.size(); ++i) {
+        auto producer = std::dynamic_pointer_cast<BinConv>(layers[i]);
+        if (!producer || !producer->fused_a || producer->output_mat->c % 64 != 0) continue;
+        for (size_t j = i + 1; j < layers.size(); ++j) {
+            auto consumer = std::dynamic_pointer_cast<BinConv>(layers[j]);
+            if (consumer && consumer->input_mat == producer->output_mat) {
+                if (consumer->method() == BinConv::DIRECT_CONV) {
+                    producer->fused_sign_out = consumer->binarized_mat;
+                    consumer->input_prepacked = true;
+                }
+                break;
+            }
+            layer_io(layers[j], rd, wr);
+            if (contains(wr, producer->output_mat.get())) break;  // the blob changes again before anyone packs it
+        }
+    }
 }
 
 void Net::run(const void *host_input) {

@@ -139,6 +139,30 @@ def bconv_3x3_affine_add(x, weight, a, b, shortcut=None, stride=1, pad=1):
     return out
 
 
+def bconv_3x3_affine_add_sign(x, weight, a, b, shortcut=None, stride=1, pad=1):
+    """bconv_3x3_affine_add that also returns pack_mat of its result (the next BinConv's packed input):
+    (fp32 [N,OH,OW,Cout], int64 [N,OH,OW,Cout/64])."""
+    _need(x, torch.int64, "x")
+    _need(weight, torch.int64, "weight")
+    _need(a, torch.float32, "a")
+    _need(b, torch.float32, "b")
+    n, h, w, cw = x.shape
+    cout = weight.shape[0]
+    if weight.numel() != cout * 9 * cw or a.numel() != cout or b.numel() != cout:
+        raise capi.DabError(capi.DAB_EINVAL, "bconv_3x3_affine_add_sign: operand sizes do not match")
+    oh, ow = out_dim(h, pad, 3, stride), out_dim(w, pad, 3, stride)
+    out = _empty((n, max(oh, 0), max(ow, 0), cout), torch.float32, x.device)
+    packed = _empty((n, max(oh, 0), max(ow, 0), max(cout // 64, 1)), torch.int64, x.device)
+    if shortcut is not None:
+        _need(shortcut, torch.float32, "shortcut")
+        if shortcut.shape != out.shape:
+            raise capi.DabError(capi.DAB_EINVAL, "bconv_3x3_affine_add_sign: shortcut shape differs from the output")
+    check(lib.dab_bconv3x3_affine_add_sign(_ptr(x), n, h, w, cw * 64, _ptr(weight), cout, stride, pad, _ptr(a), _ptr(b),
+                                           _ptr(shortcut) if shortcut is not None else None, _ptr(out), _ptr(packed),
+                                           _stream()))
+    return out, packed
+
+
 class BinConv:
     """The BinConv layer (dabnn/layers/BinConv.h:9-38, BinConv.cpp:17-191) over a batch.
 

@@ -127,6 +127,16 @@ DAB_API int dab_bconv3x3_affine_add(const uint64_t *x, int n, int h, int w, int 
                                     float *out, dab_stream_t stream);
 
 /*
+ * dab_bconv3x3_affine_add that also writes pack_mat (dabnn/bitpack.h:277-293) of its own result:
+ *   out_packed[p][c/64] bit c%64 = (out[p][c] > 0)
+ * i.e. the words BinConv::forward_impl of the next layer would make from out (dabnn/layers/BinConv.cpp:146), so
+ * that layer can skip reading the fp32 blob again.  cout must be a multiple of 64.
+ */
+DAB_API int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout,
+                                         int stride, int pad, const float *a, const float *b, const float *shortcut,
+                                         float *out, uint64_t *out_packed, dab_stream_t stream);
+
+/*
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in

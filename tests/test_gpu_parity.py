@@ -216,6 +216,35 @@ def test_bconv_affine_add_equals_three_reference_layers(dab, n, h, w, cin, cout,
     np.testing.assert_array_equal(got.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,with_shortcut", [
+    (2, 9, 7, 64, 64, 1, True), (1, 14, 14, 256, 256, 1, True), (3, 8, 8, 128, 128, 2, True), (1, 7, 7, 512, 64, 1, False),
+    (5, 13, 13, 64, 192, 1, True), (1, 56, 56, 64, 64, 1, True), (4, 7, 7, 512, 512, 1, True), (2, 14, 14, 256, 512, 2, True),
+    (3, 28, 28, 128, 128, 1, True), (70, 5, 5, 256, 64, 1, False),
+])
+def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, stride, with_shortcut):
+    """The fp32 result equals the three reference layers, and the packed copy is pack_mat of that result, bit for bit
+    (zeros, negatives and the exact-zero sums of the shortcut included)."""
+    r = rng(25)
+    cw = cin // 64
+    x = r.integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    a[::5] = 0.0  # a*cnt + b == b: constant channels, some of them exactly zero
+    b[::10] = 0.0
+    want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, 1, 1, stride, stride) for img in x])
+    sc = r.standard_normal(want.shape).astype(np.float32) if with_shortcut else None
+    for img in want:
+        orc.affine_inplace(img, a, b)
+    if with_shortcut:
+        sc[:, :, :, ::10] = 0.0
+        want = want + sc
+    got, packed = dab.bconv_3x3_affine_add_sign(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b),
+                                                dev_f(sc) if with_shortcut else None, stride, 1)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+
+
 def test_bconv_3x3_unsupported_and_invalid(dab):
     from dabnn_amd.capi import DabUnsupported
     x = torch.zeros((1, 4, 4, 3), dtype=torch.int64, device="cuda")  # 192 channels

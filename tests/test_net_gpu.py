@@ -41,6 +41,22 @@ def check_every_segment(n, layers, inits, image):
     return checked
 
 
+def check_packed_inputs(n, layers, image):
+    """The packed input every direct BinConv worked on is pack_mat of the fp32 blob it reads, whether the layer packed
+    it itself or the previous block's fused pass wrote it."""
+    checked = 0
+    descs = [d for d in n.layers() if d.startswith("Bin Conv")]
+    convs = [l for l in layers if l["type"] == "BinConv2D"]
+    assert len(descs) == len(convs)
+    for layer, desc in zip(convs, descs):
+        if "DIRECT_CONV" not in desc:
+            continue
+        packed = n.get_blob("binaized_for_%s_cal" % layer["output"])[image]
+        np.testing.assert_array_equal(packed, orc.pack_mat(n.get_blob(layer["input"])[image]), err_msg=layer["name"])
+        checked += 1
+    return checked
+
+
 def drift_ok(got, want):
     """End to end only a loose bound holds: one flipped sign early on moves the logits by about a percent."""
     assert np.corrcoef(got.ravel(), want.ravel())[0, 1] > 0.98
@@ -121,8 +137,14 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     n.run(x)
     logits = n.get_blob("logits").reshape(2, -1)
     assert logits.shape == (2, 1000)
+    descs = n.layers()
+    # every block but the first takes its packed input from the block before it; the three Adds of the down-sampling
+    # blocks are fused too, behind their shortcut branch
+    assert sum("+ Sign" in d for d in descs) == 15 and sum("packed input from the previous block" in d for d in descs) == 15
+    assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
     for i in range(2):
         assert check_every_segment(n, layers, inits, i) >= 20
+        assert check_packed_inputs(n, layers, i) == 16
     cpu = orc_net.run_model(layers, inits, x[0])
     drift_ok(logits[0], cpu["logits"])
     n.set_profile(True)
