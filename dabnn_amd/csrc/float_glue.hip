@@ -309,23 +309,22 @@ __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict
     const uint32_t img = p.div_oh.div(t2);
     const int oy = (int)(t2 - img * p.g.oh);
     float4 m = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX), sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    int cnt = 0;
     const int ys = oy * p.g.stride_h - p.g.pad_h, xs = ox * p.g.stride_w - p.g.pad_w;
-    for (int a = 0; a < p.g.kh; ++a) {
-        const int y = ys + a;
-        if ((unsigned)y >= (unsigned)p.g.h) continue;
-        const float4 *row = x + ((size_t)img * p.g.h + y) * p.g.w * p.c4 + ch;
-        for (int b = 0; b < p.g.kw; ++b) {
-            const int xx = xs + b;
-            if ((unsigned)xx >= (unsigned)p.g.w) continue;
-            const float4 v = row[(size_t)xx * p.c4];
+    // in-bounds part of the window, so that the tap loop has no branches and its loads overlap
+    const int a_lo = ys < 0 ? -ys : 0, a_hi = ys + p.g.kh > p.g.h ? p.g.h - ys : p.g.kh;
+    const int b_lo = xs < 0 ? -xs : 0, b_hi = xs + p.g.kw > p.g.w ? p.g.w - xs : p.g.kw;
+    const int cnt = (a_hi > a_lo && b_hi > b_lo) ? (a_hi - a_lo) * (b_hi - b_lo) : 0;
+    for (int a = a_lo; a < a_hi; ++a) {
+        const float4 *row = x + (((size_t)img * p.g.h + ys + a) * p.g.w + xs) * p.c4 + ch;
+#pragma unroll 8
+        for (int b = b_lo; b < b_hi; ++b) {
+            const float4 v = row[(size_t)b * p.c4];
             if (MAX) {
                 m.x = v.x > m.x ? v.x : m.x, m.y = v.y > m.y ? v.y : m.y;
                 m.z = v.z > m.z ? v.z : m.z, m.w = v.w > m.w ? v.w : m.w;
             } else {
 #pragma clang fp contract(off)
                 sum.x = sum.x + v.x, sum.y = sum.y + v.y, sum.z = sum.z + v.z, sum.w = sum.w + v.w;
-                ++cnt;
             }
         }
     }

@@ -382,7 +382,9 @@ void Net::fuse_binconv_epilogues() {
 
     for (size_t i = 0; i < layers.size(); ++i) {
         auto producer = std::dynamic_pointer_cast<BinConv>(layers[i]);
-        if (!producer || !producer->fused_a || producer->output_mat->c % 64 != 0) continue;
+        // not with 512 input channels: sign bits need work items of 8 output channels, four units there, and the
+        // coarser split costs more than the separate pack_mat it saves (measured at batch 1, 64 and 256)
+        if (!producer || !producer->fused_a || producer->output_mat->c % 64 != 0 || producer->input_mat->elem_c >= 512) continue;
         for (size_t j = i + 1; j < layers.size(); ++j) {
             auto consumer = std::dynamic_pointer_cast<BinConv>(layers[j]);
             if (consumer && consumer->input_mat == producer->output_mat) {
