@@ -81,6 +81,18 @@ __global__ __launch_bounds__(64 * kGemmWavesPerBlock, K64R >= 72 ? 3 : (K64R >= 
                 w[2 * h] = (uint32_t)v, w[2 * h + 1] = (uint32_t)(v >> 32);
             }
         }
+        // Priority by remaining work: the SIMD issues from its oldest wave first, so with equal priorities its few
+        // resident waves finish one after the other and the last one runs alone at the single-wave issue rate.
+        const int left = K64R >= 36 ? i1 - it - 1 : 0;  // 3-5 resident waves per SIMD; no effect measured with 6
+        if (left >= 3) {
+            __builtin_amdgcn_s_setprio(3);
+        } else if (left == 2) {
+            __builtin_amdgcn_s_setprio(2);
+        } else if (left == 1) {
+            __builtin_amdgcn_s_setprio(1);
+        } else {
+            __builtin_amdgcn_s_setprio(0);
+        }
         // the last run of a ragged n is shifted back so its scalar loads stay inside B
         const int j_first = run * Q;
         const int j0 = j_first + Q <= p.n ? j_first : p.n - Q;
