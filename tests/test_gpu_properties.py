@@ -116,3 +116,49 @@ def test_fused_im2col_batch64_equals_pack_of_unfold(dab):
     taps = [xp[:, a:a + 28, b:b + 28, :] for a in range(3) for b in range(3)]
     gathered = torch.cat(taps, dim=-1).reshape(-1, 9 * 128).contiguous()
     assert torch.equal(dab.pack_mat(gathered), col)
+
+
+@pytest.mark.parametrize("hw,cin,cout,stride", STAGE_SHAPES)
+def test_fused_epilogue_batch64_equals_separate_layers(dab, hw, cin, cout, stride):
+    """At full batch the one-pass BinConv + Affine + Add (+ sign) equals the separate kernels of the library bit for bit:
+    counts, then affine_inplace, add_inplace, and pack_mat of the result."""
+    gen = torch.Generator().manual_seed(7 * hw + cin + stride)
+    n = 64
+    x = rand_words(gen, n, hw, hw, cin // 64)
+    w = rand_words(gen, cout, 9 * cin // 64)
+    a = (torch.randn(cout, generator=gen) / 40).cuda()
+    b = torch.randn(cout, generator=gen).cuda()
+    a[::7] = 0.0
+    b[::14] = 0.0  # exact zeros in the result: their sign bit must be 0
+    want = dab.bconv_3x3(x, w, stride, 1)
+    sc = torch.randn(want.shape, generator=gen).cuda()
+    sc[..., ::14] = 0.0
+    dab.affine_inplace(want, a, b)
+    dab.add_inplace(want, sc)
+    got1 = dab.bconv_3x3_affine_add(x, w, a, b, sc, stride, 1)
+    assert torch.equal(got1, want)
+    got2, packed = dab.bconv_3x3_affine_add_sign(x, w, a, b, sc, stride, 1)
+    assert torch.equal(got2, want)
+    assert torch.equal(packed, dab.pack_mat(want))
+    assert (want == 0).any()
+
+
+@pytest.mark.parametrize("n,hw,c,cout,k,pad,stride", [(32, 224, 3, 64, 7, 3, 2), (16, 112, 32, 64, 3, 1, 1), (64, 28, 64, 128, 1, 0, 1),
+                                                       (256, 1, 512, 1000, 1, 0, 1), (1, 224, 3, 64, 7, 3, 2)])
+def test_fconv_full_size_against_torch(dab, n, hw, c, cout, k, pad, stride):
+    """The float convolutions of Bi-Real-18 at their real sizes against torch's fp32 convolution on the GPU, 1e-4
+    relative (the tolerance of the float layers), with and without the fused Affine + Relu."""
+    gen = torch.Generator().manual_seed(n + hw + c)
+    x = torch.randn((n, hw, hw, c), generator=gen).cuda()
+    w = (torch.randn((cout, k, k, c), generator=gen) / (k * k * c) ** 0.5).cuda()
+    bias = torch.randn(cout, generator=gen).cuda()
+    a, b = torch.randn(cout, generator=gen).cuda(), torch.randn(cout, generator=gen).cuda()
+    torch.backends.cudnn.allow_tf32 = False
+    torch.backends.cuda.matmul.allow_tf32 = False
+    ref = F.conv2d(x.permute(0, 3, 1, 2), w.permute(0, 3, 1, 2), bias, stride=stride, padding=pad).permute(0, 2, 3, 1)
+    got = dab.fconv(x, w, bias, k, k, pad, pad, stride, stride)
+    scale = ref.abs().max().item()
+    assert (got - ref).abs().max().item() <= 1e-4 * scale
+    fused = dab.fconv_affine_relu(x, w, bias, a, b, True, k, k, pad, pad, stride, stride)
+    ref2 = torch.relu(ref * a + b)
+    assert (fused - ref2).abs().max().item() <= 1e-4 * max(ref2.abs().max().item(), scale * a.abs().max().item())
