@@ -2,6 +2,8 @@
 // fconv, per-channel affine, add, average and max pooling.  All NHWC.
 #include <float.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace dab {
@@ -83,20 +85,42 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     const int l_k = tid % SK, l_r = tid / SK;
     uint32_t a_base[APT];  // byte offset of (image, y0, x0, channel 0) from the descriptor's start, modulo 2^32
     int a_y0[PADDED ? APT : 1], a_x0[PADDED ? APT : 1];
+    {
+        // the thread's first pixel by division, the others by stepping RP pixels on (one row wrap at most when the
+        // output is at least RP wide; by division again otherwise)
+        const int pix0 = m0 + l_r;
+        const uint32_t t0 = p.div_ow.div((uint32_t)pix0);
+        int ox = pix0 - (int)t0 * p.ow;
+        int img = (int)p.div_oh.div(t0);
+        int oy = (int)t0 - img * p.oh;
+        const bool step_ok = p.ow >= RP;
 #pragma unroll
-    for (int i = 0; i < APT; ++i) {
-        const int pix = m0 + l_r + RP * i;
-        if (pix < p.M) {
-            const uint32_t t = p.div_ow.div((uint32_t)pix);
-            const int ox = pix - (int)t * p.ow;
-            const int img = (int)p.div_oh.div(t);
-            const int oy = (int)t - img * p.oh;
-            const int y0 = oy * p.stride_h - p.pad_h, x0 = ox * p.stride_w - p.pad_w;
-            a_base[i] = (uint32_t)((((img - img0) * p.h + y0) * p.wd + x0) * p.c) * 4u;
-            if (PADDED) a_y0[i] = y0, a_x0[i] = x0;
-        } else {
-            a_base[i] = kOobRow;
-            if (PADDED) a_y0[i] = -(1 << 30), a_x0[i] = 0;  // every tap fails the bounds test
+        for (int i = 0; i < APT; ++i) {
+            const int pix = pix0 + RP * i;
+            if (i > 0) {
+                if (step_ok) {
+                    ox += RP;
+                    const bool wrap = ox >= p.ow;
+                    ox = wrap ? ox - p.ow : ox;
+                    oy += wrap ? 1 : 0;
+                    const bool wrap2 = oy >= p.oh;
+                    oy = wrap2 ? 0 : oy;
+                    img += wrap2 ? 1 : 0;
+                } else {
+                    const uint32_t t = p.div_ow.div((uint32_t)pix);
+                    ox = pix - (int)t * p.ow;
+                    img = (int)p.div_oh.div(t);
+                    oy = (int)t - img * p.oh;
+                }
+            }
+            if (pix < p.M) {
+                const int y0 = oy * p.stride_h - p.pad_h, x0 = ox * p.stride_w - p.pad_w;
+                a_base[i] = (uint32_t)((((img - img0) * p.h + y0) * p.wd + x0) * p.c) * 4u;
+                if (PADDED) a_y0[i] = y0, a_x0[i] = x0;
+            } else {
+                a_base[i] = kOobRow;
+                if (PADDED) a_y0[i] = -(1 << 30), a_x0[i] = 0;  // every tap fails the bounds test
+            }
         }
     }
     uint32_t b_row[BPT];
@@ -172,52 +196,73 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
         __syncthreads();
     }
 
-    // row: tile row of the output element; rows past the last pixel are past the end of the output descriptor
-    auto emit = [&](int row, uint32_t co_off, float v, float bias, float fa, float fb) {
+    // Epilogue.  The three optional steps are decided once per launch, so the per-element code is straight-line:
+    // (+ bias) (a*v + b, two roundings) (relu) and one store.  An element's byte offset is the lane's own part (its
+    // column, its share of the row index) plus a wave-uniform multiple of the row pitch; rows past the last pixel are
+    // past the end of the output descriptor and a column past the last channel carries kOob.
+    const uint32_t row_bytes = (uint32_t)p.cout * 4u;
+    auto emit = [&](auto has_bias, auto has_affine, auto has_relu, uint32_t off, float v, float bias, float fa, float fb) {
 #pragma clang fp contract(off)
-        if (p.bias) v = v + bias;
-        if (p.aff_a) {
+        if constexpr (decltype(has_bias)::value) v = v + bias;
+        if constexpr (decltype(has_affine)::value) {
             const float prod = fa * v;
             v = prod + fb;
         }
-        if (p.relu) v = v > 0.f ? v : 0.f;
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), o_rsrc,
-                                              (int)((uint32_t)row * p.cout * 4u + co_off), 0, 0);
+        if constexpr (decltype(has_relu)::value) v = v > 0.f ? v : 0.f;
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), o_rsrc, (int)off, 0, 0);
     };
-
     // accumulator element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l % 32
-    if (KSPLIT == 1) {
+    auto emit_all = [&](auto has_bias, auto has_affine, auto has_relu) {
+        if constexpr (KSPLIT == 1) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const int co = n0 + wn * WTN + j * 32 + f_i;
+            for (int j = 0; j < TN; ++j) {
+                const int co = n0 + wn * WTN + j * 32 + f_i;
+                const bool co_ok = co < p.cout;
+                const float bias = (decltype(has_bias)::value && co_ok) ? p.bias[co] : 0.f;
+                const float fa = (decltype(has_affine)::value && co_ok) ? p.aff_a[co] : 0.f;
+                const float fb = (decltype(has_affine)::value && co_ok) ? p.aff_b[co] : 0.f;
+                const uint32_t lane_off = (co_ok ? (uint32_t)co * 4u : kOob) + (uint32_t)(wm * WTM + 4 * f_k) * row_bytes;
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        emit(has_bias, has_affine, has_relu, lane_off + (uint32_t)(i * 32 + 8 * (e / 4) + (e % 4)) * row_bytes,
+                             acc[i][j][e], bias, fa, fb);
+            }
+        } else {
+            // one 32 x 32 tile: the waves' partial sums are added in wave order, four accumulator elements per thread
+            const int co = n0 + f_i;
             const bool co_ok = co < p.cout;
-            const float bias = (p.bias && co_ok) ? p.bias[co] : 0.f;
-            const float fa = (p.aff_a && co_ok) ? p.aff_a[co] : 0.f, fb = (p.aff_a && co_ok) ? p.aff_b[co] : 0.f;
-            const uint32_t co_off = co_ok ? (uint32_t)co * 4u : kOob;
+            const float bias = (decltype(has_bias)::value && co_ok) ? p.bias[co] : 0.f;
+            const float fa = (decltype(has_affine)::value && co_ok) ? p.aff_a[co] : 0.f;
+            const float fb = (decltype(has_affine)::value && co_ok) ? p.aff_b[co] : 0.f;
+            const uint32_t lane_off = (co_ok ? (uint32_t)co * 4u : kOob) + (uint32_t)(4 * f_k) * row_bytes;
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+            for (int q = 0; q < 16 / KSPLIT; ++q) {
+                const int e = wave * (16 / KSPLIT) + q;
+                float v = red[e * 64 + lane];
 #pragma unroll
-                for (int e = 0; e < 16; ++e)
-                    emit(wm * WTM + i * 32 + 8 * (e / 4) + 4 * f_k + (e % 4), co_off, acc[i][j][e], bias, fa, fb);
+                for (int s = 1; s < KSPLIT; ++s) v = __fadd_rn(v, red[(s * 16 + e) * 64 + lane]);
+                emit(has_bias, has_affine, has_relu, lane_off + (uint32_t)(8 * (e / 4) + (e % 4)) * row_bytes, v, bias, fa, fb);
+            }
         }
-    } else {
-        // one 32 x 32 tile: the waves' partial sums are added in wave order, four accumulator elements per thread
+    };
+    if constexpr (KSPLIT > 1) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) red[(ks * 16 + e) * 64 + lane] = acc[0][0][e];
         __syncthreads();
-        const int co = n0 + f_i;
-        const bool co_ok = co < p.cout;
-        const float bias = (p.bias && co_ok) ? p.bias[co] : 0.f;
-        const float fa = (p.aff_a && co_ok) ? p.aff_a[co] : 0.f, fb = (p.aff_a && co_ok) ? p.aff_b[co] : 0.f;
-        const uint32_t co_off = co_ok ? (uint32_t)co * 4u : kOob;
-#pragma unroll
-        for (int q = 0; q < 16 / KSPLIT; ++q) {
-            const int e = wave * (16 / KSPLIT) + q;
-            float v = red[e * 64 + lane];
-#pragma unroll
-            for (int s = 1; s < KSPLIT; ++s) v = __fadd_rn(v, red[(s * 16 + e) * 64 + lane]);
-            emit(8 * (e / 4) + 4 * f_k + (e % 4), co_off, v, bias, fa, fb);
-        }
+    }
+    using T = std::true_type;
+    using F = std::false_type;
+    switch ((p.bias ? 4 : 0) | (p.aff_a ? 2 : 0) | (p.relu ? 1 : 0)) {
+        case 0: emit_all(F{}, F{}, F{}); break;
+        case 1: emit_all(F{}, F{}, T{}); break;
+        case 2: emit_all(F{}, T{}, F{}); break;
+        case 3: emit_all(F{}, T{}, T{}); break;
+        case 4: emit_all(T{}, F{}, F{}); break;
+        case 5: emit_all(T{}, F{}, T{}); break;
+        case 6: emit_all(T{}, T{}, F{}); break;
+        default: emit_all(T{}, T{}, T{}); break;
     }
 }
 
