@@ -136,8 +136,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
             __builtin_amdgcn_s_setprio(0);
         }
         uint32_t acc[Q];
-#pragma unroll
-        for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
         unit_rowmajor<K32, Q, (CW >= 2 ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
         const int slot = cg % WU;
         stage_put<WCH, Q>(stage, lane, slot * Q, acc);

@@ -97,8 +97,6 @@ __global__ __launch_bounds__(64 * kGemmWavesPerBlock, K64R >= 72 ? 3 : (K64R >= 
         const int j_first = run * Q;
         const int j0 = j_first + Q <= p.n ? j_first : p.n - Q;
         uint32_t acc[Q];
-#pragma unroll
-        for (int q = 0; q < Q; ++q) acc[q] = kAccInit;
         unit_rowmajor<K32, Q, 2>(p.b + (size_t)j0 * K64R, w, acc);  // B streams through the scalar cache: two vectors per wait
         add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
         if (++run == p.n_runs) {

@@ -73,6 +73,19 @@ __device__ __forceinline__ void xp2(uint32_t &acc, uint32_t w0, uint32_t w1, uin
         : "s"(w0), "s"(w1), "v"(a0), "v"(a1));
 }
 
+// The same for the first dword pair of a channel: acc = init + popcount(..) + popcount(..), init in an SGPR, so the
+// accumulator needs no separate initialisation.
+__device__ __forceinline__ void xp2_first(uint32_t &acc, uint32_t init, uint32_t w0, uint32_t w1, uint32_t a0, uint32_t a1) {
+    uint32_t t0, t1;
+    asm volatile(
+        "v_xor_b32 %1, %3, %5\n\t"
+        "v_xor_b32 %2, %4, %6\n\t"
+        "v_bcnt_u32_b32 %0, %1, %7\n\t"
+        "v_bcnt_u32_b32 %0, %2, %0"
+        : "=&v"(acc), "=&v"(t0), "=&v"(t1)
+        : "s"(w0), "s"(w1), "v"(a0), "v"(a1), "s"(init));
+}
+
 // Accumulators start at the bit pattern of 2^23: adding an integer count
 // c < 2^23 to that pattern yields the float 2^23 + c exactly, so one
 // subtraction replaces the integer-to-float conversion.
@@ -92,6 +105,7 @@ constexpr int kMaxCount = (1 << 23) - 1;
 // so the latency cover of a batch is the vector work of the previous one: one
 // vector (32 vector instructions) covers a scalar-cache hit, two ride out a
 // miss to L2 (operands too large for the 16 KiB scalar cache).
+// acc is an output: acc[q] = 2^23 pattern + mismatch count of channel q.
 template <int K32, int Q, int BV_WANTED = 1>
 __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[Q]) {
     constexpr int D = Q * K32;
@@ -101,6 +115,7 @@ __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t 
     constexpr int NB = NV / BV;
     static_assert(K32 % 2 == 0 && D % VW == 0, "a dword pair never straddles two channels");
     typename SVec<VW>::type buf[2][BV];
+    const uint32_t acc_init = kAccInit;  // the accumulators are written, not updated, by each channel's first pair
     static_for<BV>([&](auto b_) { sload<VW, b_ * VW * 4>(buf[0][b_], wbase); });
     static_for<BV>([&](auto b_) { swait(buf[0][b_]); });
     static_for<NB>([&](auto j_) {
@@ -111,7 +126,10 @@ __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t 
             static_for<VW / 2>([&](auto e_) {
                 constexpr int d = (j * BV + b_) * VW + e_ * 2;  // dword index within the Q-channel block
                 constexpr int q = d / K32, k = d % K32;
-                xp2(acc[q], buf[j & 1][b_][e_ * 2], buf[j & 1][b_][e_ * 2 + 1], a[k], a[k + 1]);
+                if constexpr (k == 0)
+                    xp2_first(acc[q], acc_init, buf[j & 1][b_][e_ * 2], buf[j & 1][b_][e_ * 2 + 1], a[k], a[k + 1]);
+                else
+                    xp2(acc[q], buf[j & 1][b_][e_ * 2], buf[j & 1][b_][e_ * 2 + 1], a[k], a[k + 1]);
             });
         });
         if constexpr (j + 1 < NB) static_for<BV>([&](auto b_) { swait(buf[(j + 1) & 1][b_]); });
