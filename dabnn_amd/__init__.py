@@ -22,6 +22,7 @@ from .ops import (  # noqa: F401
     fconv_affine_relu,
     fused_binarize_im2col,
     max_pool,
+    max_pool_sign,
     pack_mat,
     pad,
     weight_transpose,

@@ -63,6 +63,7 @@ SIGNATURES = {
     "dab_fill_f32": (_i, [_vp, _i64, ctypes.c_float, _vp]),
     "dab_ave_pool": (_i, [_vp] + [_i] * 10 + [_vp, _vp]),
     "dab_max_pool": (_i, [_vp] + [_i] * 10 + [_vp, _vp]),
+    "dab_max_pool_sign": (_i, [_vp] + [_i] * 10 + [_vp, _vp, _vp]),
 }
 
 for _name, (_res, _args) in SIGNATURES.items():

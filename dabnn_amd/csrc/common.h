@@ -71,6 +71,17 @@ struct FastDiv {
     __device__ __forceinline__ uint32_t div(uint32_t n) const { return d == 1 ? n : (__umulhi(n, mul) >> shift); }
 };
 
+// ---------------------------------------------------------------- sign bits of results
+// Bit i = (component i > 0): the packing rule of pack_64 (common/common_bitpack.h:12-34) for four channels.
+__device__ __forceinline__ uint32_t sign_nibble(float4 r) {
+    return (uint32_t)(r.x > 0.0f) | ((uint32_t)(r.y > 0.0f) << 1) | ((uint32_t)(r.z > 0.0f) << 2) | ((uint32_t)(r.w > 0.0f) << 3);
+}
+// v | (v of lane + N within the row of 16 lanes; zero past the row's end): DPP row_shl:N
+template <int N>
+__device__ __forceinline__ uint32_t or_from_lane_above(uint32_t v) {
+    return v | (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x100 + N, 0xF, 0xF, true);
+}
+
 // ---------------------------------------------------------------- buffer resources
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

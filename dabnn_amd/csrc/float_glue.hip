@@ -342,9 +342,11 @@ struct PoolVecArgs {
     FastDiv div_c4, div_ow, div_oh;
 };
 
-template <bool MAX>
+// SIGN (c % 64 == 0): the 16 threads that hold the 64 channels of a word are one row of lanes; their sign nibbles are
+// gathered with DPP and the first of them stores pack_mat's word of the pooled pixel (dabnn/bitpack.h:277-293).
+template <bool MAX, bool SIGN>
 __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict__ x, float4 *__restrict__ out,
-                                                        const PoolVecArgs p) {
+                                                        uint64_t *__restrict__ out_packed, const PoolVecArgs p) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
     if (idx >= p.total) return;
     uint32_t t = p.div_c4.div(idx);
@@ -373,11 +375,24 @@ __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict
             }
         }
     }
+    float4 r;
     if (MAX) {
-        out[idx] = m;
+        r = m;
     } else {
         const float d = (float)cnt;
-        out[idx] = make_float4(__fdiv_rn(sum.x, d), __fdiv_rn(sum.y, d), __fdiv_rn(sum.z, d), __fdiv_rn(sum.w, d));
+        r = make_float4(__fdiv_rn(sum.x, d), __fdiv_rn(sum.y, d), __fdiv_rn(sum.z, d), __fdiv_rn(sum.w, d));
+    }
+    out[idx] = r;
+    if constexpr (SIGN) {
+        // total is a multiple of 16 here, so a row of lanes is either complete or has returned above as a whole
+        const int part = (int)(idx & 15u);
+        const uint32_t nib = sign_nibble(r);
+        uint32_t lo = part < 8 ? nib << (4 * part) : 0u, hi = part >= 8 ? nib << (4 * (part - 8)) : 0u;
+        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+        if (part == 0) out_packed[idx >> 4] = ((uint64_t)hi << 32) | lo;
     }
 }
 
@@ -505,9 +520,9 @@ extern "C" int dab_fill_f32(float *x, int64_t n_elem, float value, dab_stream_t 
 }
 
 static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
-                       int stride_h, int stride_w, float *out, dab_stream_t stream) {
+                       int stride_h, int stride_w, float *out, uint64_t *out_packed, bool want_sign, dab_stream_t stream) {
     using namespace dab;
-    DAB_REQUIRE(x && out, "dab_pool: null pointer");
+    DAB_REQUIRE(x && out && (out_packed || !want_sign), "dab_pool: null pointer");
     DAB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && kh > 0 && kw > 0, "dab_pool: non-positive dimension");
     DAB_REQUIRE(pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0, "dab_pool: bad pad/stride");
     PoolArgs a;
@@ -517,17 +532,26 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
     a.oh = out_dim(h, pad_h, kh, 1, stride_h), a.ow = out_dim(w, pad_w, kw, 1, stride_w);
     DAB_REQUIRE(a.oh > 0 && a.ow > 0, "dab_pool: empty output");
     const long long total = (long long)n * a.oh * a.ow * c;
-    if (c % 4 == 0 && total / 4 < (1ll << 31) - 256 && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 == 0) {
+    const bool vec_ok = c % 4 == 0 && total / 4 < (1ll << 31) - 256 &&
+                        (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % 16 == 0;
+    if (want_sign) {
+        if (c % 64 != 0 || !vec_ok || !is_max)
+            return fail(DAB_EUNSUPPORTED, "dab_max_pool_sign: needs c %% 64 == 0, 16-byte aligned buffers and fewer than 2^33 outputs");
+        DAB_REQUIRE(reinterpret_cast<uintptr_t>(out_packed) % 8 == 0, "dab_max_pool_sign: misaligned packed output");
+    }
+    if (vec_ok) {
         PoolVecArgs v;
         v.g = a, v.c4 = c / 4, v.total = (uint32_t)(total / 4);
         v.div_c4 = FastDiv((uint32_t)v.c4), v.div_ow = FastDiv((uint32_t)a.ow), v.div_oh = FastDiv((uint32_t)a.oh);
         const unsigned vb = (v.total + 255u) / 256u;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         float4 *o4 = reinterpret_cast<float4 *>(out);
-        if (is_max)
-            hipLaunchKernelGGL(pool_vec4_kernel<true>, dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, v);
+        if (want_sign)
+            hipLaunchKernelGGL((pool_vec4_kernel<true, true>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, out_packed, v);
+        else if (is_max)
+            hipLaunchKernelGGL((pool_vec4_kernel<true, false>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, nullptr, v);
         else
-            hipLaunchKernelGGL(pool_vec4_kernel<false>, dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, v);
+            hipLaunchKernelGGL((pool_vec4_kernel<false, false>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, nullptr, v);
         DAB_LAUNCH_CHECK();
         return DAB_OK;
     }
@@ -542,10 +566,15 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
 
 extern "C" int dab_ave_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
                             int stride_h, int stride_w, float *out, dab_stream_t stream) {
-    return pool_common(false, x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, out, stream);
+    return pool_common(false, x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, out, nullptr, false, stream);
 }
 
 extern "C" int dab_max_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
                             int stride_h, int stride_w, float *out, dab_stream_t stream) {
-    return pool_common(true, x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, out, stream);
+    return pool_common(true, x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, out, nullptr, false, stream);
+}
+
+extern "C" int dab_max_pool_sign(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                                 int stride_h, int stride_w, float *out, uint64_t *out_packed, dab_stream_t stream) {
+    return pool_common(true, x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, out, out_packed, true, stream);
 }

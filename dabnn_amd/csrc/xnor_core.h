@@ -240,14 +240,6 @@ struct EpiAffineAddSign : EpiAffineAdd {
     int bits_ld;          // cout / 8
 };
 
-__device__ __forceinline__ uint32_t sign_nibble(float4 r) {
-    return (uint32_t)(r.x > 0.0f) | ((uint32_t)(r.y > 0.0f) << 1) | ((uint32_t)(r.z > 0.0f) << 2) | ((uint32_t)(r.w > 0.0f) << 3);
-}
-// v | (v of lane + N within the row of 16 lanes; zero past the row's end): DPP row_shl:N
-template <int N>
-__device__ __forceinline__ uint32_t or_from_lane_above(uint32_t v) {
-    return v | (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x100 + N, 0xF, 0xF, true);
-}
 
 // Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
 // WCH-channel window that starts at channel cbase.  out is [pixel][ld] floats;

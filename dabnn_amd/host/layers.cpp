@@ -128,7 +128,7 @@ std::string BinConv::to_str() const {
     ss << type_ << ", input " << input_mat->h << "x" << input_mat->w << "x" << input_mat->elem_c << ", weight "
        << weight_mat->n << "x" << kernel_h() << "x" << kernel_w() << ", pad " << pad_h << "," << pad_w << ", stride "
        << stride_h << "," << stride_w << ", method " << (method() == DIRECT_CONV ? "DIRECT_CONV" : "BGEMM");
-    if (input_prepacked) ss << ", packed input from the previous block";
+    if (input_prepacked) ss << ", packed input from its producer";
     if (fused_a) ss << (fused_shortcut ? " + Affine + Add" : " + Affine");
     if (fused_sign_out) ss << " + Sign";
     return ss.str();
@@ -240,6 +240,13 @@ MaxPool::MaxPool(NetCP net, css name, css input, css output, int kernel_h_, int 
       stride_w(stride_w_) {}
 
 void MaxPool::forward_impl() const {
+    if (fused_sign_out) {
+        dab_check(dab_max_pool_sign(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+                                    input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
+                                    static_cast<float *>(output_mat->data), static_cast<uint64_t *>(fused_sign_out->data),
+                                    stream()));
+        return;
+    }
     dab_check(dab_max_pool(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
                            input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
                            static_cast<float *>(output_mat->data), stream()));

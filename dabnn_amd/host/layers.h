@@ -88,6 +88,8 @@ class AvePool : public Layer {
 class MaxPool : public Layer {
    public:
     MatP input_mat, output_mat;
+    // Set by Net::prepare when a direct BinConv reads the pooled blob: its packed input, written in the same pass.
+    MatP fused_sign_out;
     const int kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w;
     MaxPool(NetCP net, css name, css input, css output, int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h,
             int stride_w);

@@ -380,6 +380,23 @@ void Net::fuse_binconv_epilogues() {
     }
     layers.swap(out);
 
+    // the same for a MaxPool whose output a direct BinConv packs (the first block of a Bi-Real net)
+    for (size_t i = 0; i < layers.size(); ++i) {
+        auto pool = std::dynamic_pointer_cast<MaxPool>(layers[i]);
+        if (!pool || pool->output_mat->c % 64 != 0) continue;
+        for (size_t j = i + 1; j < layers.size(); ++j) {
+            auto consumer = std::dynamic_pointer_cast<BinConv>(layers[j]);
+            if (consumer && consumer->input_mat == pool->output_mat) {
+                if (consumer->method() == BinConv::DIRECT_CONV && !consumer->input_prepacked) {
+                    pool->fused_sign_out = consumer->binarized_mat;
+                    consumer->input_prepacked = true;
+                }
+                break;
+            }
+            layer_io(layers[j], rd, wr);
+            if (contains(wr, pool->output_mat.get())) break;
+        }
+    }
     for (size_t i = 0; i < layers.size(); ++i) {
         auto producer = std::dynamic_pointer_cast<BinConv>(layers[i]);
         // not with 512 input channels: sign bits need work items of 8 output channels, four units there, and the

@@ -278,3 +278,15 @@ def ave_pool(x, kh, kw, pad_h, pad_w, stride_h, stride_w):
 def max_pool(x, kh, kw, pad_h, pad_w, stride_h, stride_w):
     """max_pool_fallback (dabnn/layers/MaxPool.cpp:209-246)."""
     return _pool(lib.dab_max_pool, x, kh, kw, pad_h, pad_w, stride_h, stride_w)
+
+
+def max_pool_sign(x, kh, kw, pad_h, pad_w, stride_h, stride_w):
+    """max_pool that also returns pack_mat of its result: (fp32 [N,OH,OW,C], int64 [N,OH,OW,C/64])."""
+    _need(x, torch.float32, "x")
+    n, h, w, c = x.shape
+    oh, ow = out_dim(h, pad_h, kh, stride_h), out_dim(w, pad_w, kw, stride_w)
+    out = _empty((n, max(oh, 0), max(ow, 0), c), torch.float32, x.device)
+    packed = _empty((n, max(oh, 0), max(ow, 0), max(c // 64, 1)), torch.int64, x.device)
+    check(lib.dab_max_pool_sign(_ptr(x), n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, _ptr(out), _ptr(packed),
+                                _stream()))
+    return out, packed

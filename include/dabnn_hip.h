@@ -194,6 +194,14 @@ DAB_API int dab_ave_pool(const float *x, int n, int h, int w, int c, int kh, int
 DAB_API int dab_max_pool(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
                  int stride_w, float *out, dab_stream_t stream);
 
+/*
+ * dab_max_pool that also writes pack_mat (dabnn/bitpack.h:277-293) of its result, the packed input of a BinConv that
+ * reads the pooled blob (the first block of a Bi-Real net): out_packed[p][c/64] bit c%64 = (out[p][c] > 0).
+ * c must be a multiple of 64, x and out 16-byte aligned.
+ */
+DAB_API int dab_max_pool_sign(const float *x, int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                              int stride_h, int stride_w, float *out, uint64_t *out_packed, dab_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -354,6 +354,19 @@ def test_fconv_ramp_cases_of_reference_tests(dab):
         np.testing.assert_array_equal(got, orc.baseline_fconv(x[0], wgt, k, k, pad, pad, stride, stride))
 
 
+@pytest.mark.parametrize("n,h,w,c,k,pad,stride", [(1, 9, 6, 64, 3, 1, 2), (2, 112, 112, 64, 3, 1, 2), (3, 7, 7, 192, 2, 0, 2),
+                                                  (1, 5, 5, 128, 3, 1, 1)])
+def test_max_pool_sign_packs_its_own_output(dab, n, h, w, c, k, pad, stride):
+    x = special_floats((n, h, w, c), 44)
+    x[np.isnan(x)] = 0.0  # the reference's max over NaN depends on the tap order; zeros and infinities stay
+    got, packed = dab.max_pool_sign(dev_f(x), k, k, pad, pad, stride, stride)
+    want = np.stack([orc.max_pool(img, k, k, pad, pad, stride, stride) for img in x])
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+    with pytest.raises(RuntimeError):
+        dab.max_pool_sign(torch.zeros((1, 4, 4, 32), device="cuda"), 2, 2, 0, 0, 2, 2)
+
+
 def test_affine_add_bit_exact(dab):
     r = rng(41)
     x = r.standard_normal((2, 5, 7, 64)).astype(np.float32)

@@ -138,9 +138,10 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     logits = n.get_blob("logits").reshape(2, -1)
     assert logits.shape == (2, 1000)
     descs = n.layers()
-    # every block up to the first one with 512 input channels hands its successor the packed input; the three Adds of the down-sampling
+    # the max pool and every block up to the first one with 512 input channels hand their successor the packed input;
+    # the three Adds of the down-sampling
     # blocks are fused too, behind their shortcut branch
-    assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from the previous block" in d for d in descs) == 13
+    assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from its producer" in d for d in descs) == 14
     assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
     for i in range(2):
         assert check_every_segment(n, layers, inits, i) >= 20
