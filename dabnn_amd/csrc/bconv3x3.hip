@@ -56,18 +56,22 @@ constexpr int kModeCounts = 0, kModeAffineAdd = 1, kModeAffineAddSign = 2;
 // Resident waves per SIMD the kernel is built for, and the staging window that lets them fit the CU's LDS:
 // the activations take 18*CW VGPRs, so 64 and 128 channels leave room for 8 and 6 waves (with the 16-channel
 // window, 5 KB per wave), 256 channels for 4 and 512 channels (144 of 512/3 = 168 VGPRs) for 3.
-template <int CW>
+// 64 channels have a second build (NARROW): 4 waves, the 32-channel window (whole 128-byte lines, no extra write
+// traffic) and wave priorities.  Measured at batch 64: faster when a wave gets 4 units or more (56x56 64->64:
+// 17.2 against 18.4 us), slower when it gets fewer (56x56 -> 28x28 64->128: 11.2 against 10.2 us).
+template <int CW, bool NARROW>
 struct Residency {
-    static constexpr int waves_per_simd = CW == 1 ? 8 : CW == 2 ? 6 : CW == 4 ? 4 : 3;
-    static constexpr int window = CW <= 2 ? 16 : 32;
+    static constexpr int waves_per_simd = NARROW ? 4 : (CW == 1 ? 8 : CW == 2 ? 6 : CW == 4 ? 4 : 3);
+    static constexpr int window = (CW <= 2 && !NARROW) ? 16 : 32;
+    static constexpr bool priorities = waves_per_simd <= 4;
 };
 
-template <int CW, int MODE>
-__global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd) void bconv3x3_kernel(const BconvArgs p) {
+template <int CW, int MODE, bool NARROW>
+__global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_per_simd)) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
     constexpr int Q = UnitChannels<CW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
-    constexpr int WCH = Residency<CW>::window;
+    constexpr int WCH = Residency<CW, NARROW>::window;
     constexpr int WU = WCH / Q;  // units per staging window
     constexpr int kStageBytes = Stage<WCH>::bytes;
     __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
@@ -124,8 +128,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
 
         // The SIMD issues from its oldest wave first, so with equal priorities the waves of a SIMD finish one after
         // the other and the last one runs alone at the single-wave issue rate.  Priority by remaining work keeps
-        // them level: they reach their last units together.
-        const int left = CW >= 4 ? u1 - u - 1 : 0;  // measured: no gain with 7-8 resident waves per SIMD
+        // them level: they reach their last units together.  (No gain measured with 7-8 resident waves.)
+        const int left = Residency<CW, NARROW>::priorities ? u1 - u - 1 : 0;
         if (left >= 3) {
             __builtin_amdgcn_s_setprio(3);
         } else if (left == 2) {
@@ -169,21 +173,31 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, Residency<CW>::waves_per_simd)
     }
 }
 
-template <int CW, int MODE>
-static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
+template <int CW, int MODE, bool NARROW>
+static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE>, 64 * kWavesPerBlock);
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW>, 64 * kWavesPerBlock);
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
     a.div_groups = FastDiv((uint32_t)a.n_groups);
-    hipLaunchKernelGGL((bconv3x3_kernel<CW, MODE>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
+    hipLaunchKernelGGL((bconv3x3_kernel<CW, MODE, NARROW>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
+}
+
+template <int CW, int MODE>
+static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
+    if constexpr (CW == 1) {
+        // four units or more per wave at four waves per SIMD
+        const long long units = tiles * (a.cout / UnitChannels<1>::value);
+        if (units >= 4ll * simd_count() * 4) return launch_variant<1, MODE, true>(a, tiles, stream);
+    }
+    return launch_variant<CW, MODE, false>(a, tiles, stream);
 }
 
 }  // namespace dab
