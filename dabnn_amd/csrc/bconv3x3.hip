@@ -56,9 +56,10 @@ constexpr int kModeCounts = 0, kModeAffineAdd = 1, kModeAffineAddSign = 2;
 // Resident waves per SIMD the kernel is built for, and the staging window that lets them fit the CU's LDS:
 // the activations take 18*CW VGPRs, so 64 and 128 channels leave room for 8 and 6 waves (with the 16-channel
 // window, 5 KB per wave), 256 channels for 4 and 512 channels (144 of 512/3 = 168 VGPRs) for 3.
-// 64 channels have a second build (NARROW): 4 waves, the 32-channel window (whole 128-byte lines, no extra write
-// traffic) and wave priorities.  Measured at batch 64: faster when a wave gets 4 units or more (56x56 64->64:
-// 17.2 against 18.4 us), slower when it gets fewer (56x56 -> 28x28 64->128: 11.2 against 10.2 us).
+// 64 and 128 channels have a second build (NARROW): 4 waves, the 32-channel window (whole 128-byte lines, no extra
+// write traffic) and wave priorities.  Measured: faster when a wave gets enough units (64 channels, 6 per wave:
+// 17.2 against 18.4 us; 128 channels, 12 per wave: 51 against 55 us), slower when it gets few (64 channels, 3 per
+// wave: 11.2 against 10.2 us; 128 channels, 3 per wave: 17.3 against 16.1 us).
 template <int CW, bool NARROW>
 struct Residency {
     static constexpr int waves_per_simd = NARROW ? 4 : (CW == 1 ? 8 : CW == 2 ? 6 : CW == 4 ? 4 : 3);
@@ -192,10 +193,10 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
-    if constexpr (CW == 1) {
-        // four units or more per wave at four waves per SIMD
-        const long long units = tiles * (a.cout / UnitChannels<1>::value);
-        if (units >= 4ll * simd_count() * 4) return launch_variant<1, MODE, true>(a, tiles, stream);
+    if constexpr (CW <= 2) {
+        // four (eight) units or more per wave at four waves per SIMD
+        const long long units = tiles * (a.cout / UnitChannels<CW>::value);
+        if (units >= (CW == 1 ? 4ll : 8ll) * simd_count() * 4) return launch_variant<CW, MODE, true>(a, tiles, stream);
     }
     return launch_variant<CW, MODE, false>(a, tiles, stream);
 }
