@@ -18,6 +18,7 @@ from .ops import (  # noqa: F401
     bgemm,
     bitpack_nchw,
     col_row_words,
+    concat,
     fconv,
     fconv_affine_relu,
     fused_binarize_im2col,
@@ -25,5 +26,7 @@ from .ops import (  # noqa: F401
     max_pool_sign,
     pack_mat,
     pad,
+    prelu_inplace,
+    relu_inplace,
     weight_transpose,
 )

@@ -290,6 +290,28 @@ __global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, long l
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = x[i] > 0.f ? x[i] : 0.f;
 }
 
+// PRelu.cpp:6-30: negative values are scaled by one slope or by their channel's slope (slope_n = 1 or c).
+__global__ __launch_bounds__(256) void prelu_kernel(float *__restrict__ x, long long total, int c,
+                                                    const float *__restrict__ slope, int slope_n) {
+    const long long stride = (long long)gridDim.x * 256;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        const float v = x[i];
+        if (v < 0.f) x[i] = v * slope[slope_n == 1 ? 0 : (int)(i % c)];
+    }
+}
+
+// Concat.cpp:7-21: per pixel the ca floats of a, then the cb floats of b.
+__global__ __launch_bounds__(256) void concat_kernel(const float *__restrict__ a, int ca, const float *__restrict__ b, int cb,
+                                                     float *__restrict__ out, long long total) {
+    const long long stride = (long long)gridDim.x * 256;
+    const int c = ca + cb;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        const long long pix = i / c;
+        const int ch = (int)(i - pix * c);
+        out[i] = ch < ca ? a[pix * ca + ch] : b[pix * cb + (ch - ca)];
+    }
+}
+
 __global__ __launch_bounds__(256) void fill_kernel(float *__restrict__ x, long long total, float v) {
     const long long stride = (long long)gridDim.x * 256;
     for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = v;
@@ -508,6 +530,29 @@ extern "C" int dab_relu_inplace(float *x, int64_t n_elem, dab_stream_t stream) {
     DAB_REQUIRE(x, "dab_relu_inplace: null pointer");
     DAB_REQUIRE(n_elem > 0, "dab_relu_inplace: n_elem %lld", (long long)n_elem);
     hipLaunchKernelGGL(relu_kernel, dim3(grid_for(n_elem)), dim3(256), 0, as_stream(stream), x, (long long)n_elem);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_prelu_inplace(float *x, int64_t n_pix, int c, const float *slope, int slope_n, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && slope, "dab_prelu_inplace: null pointer");
+    DAB_REQUIRE(n_pix > 0 && c > 0, "dab_prelu_inplace: n_pix %lld c %d", (long long)n_pix, c);
+    DAB_REQUIRE(slope_n == 1 || slope_n == c, "dab_prelu_inplace: slope must have size 1 or c (%d), got %d", c, slope_n);
+    const long long total = (long long)n_pix * c;
+    hipLaunchKernelGGL(prelu_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), x, total, c, slope, slope_n);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_concat_channels(const float *a, int ca, const float *b, int cb, int64_t n_pix, float *out,
+                                   dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(a && b && out, "dab_concat_channels: null pointer");
+    DAB_REQUIRE(n_pix > 0 && ca > 0 && cb > 0, "dab_concat_channels: n_pix %lld ca %d cb %d", (long long)n_pix, ca, cb);
+    DAB_REQUIRE(out != a && out != b, "dab_concat_channels: out must not alias an input");
+    const long long total = (long long)n_pix * (ca + cb);
+    hipLaunchKernelGGL(concat_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), a, ca, b, cb, out, total);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }

@@ -208,6 +208,33 @@ void Relu::forward_impl() const {
     dab_check(dab_relu_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->total(), stream()));
 }
 
+// dabnn/layers/PRelu.cpp:6-30; the size check is the reference's, made once at construction
+PRelu::PRelu(NetCP net, css name, css data, css slope)
+    : Layer(net, name, "PRelu"), data_mat(mat(data)), slope_mat(mat(slope)) {
+    BNN_ASSERT(slope_mat->total() == 1 || (int)slope_mat->total() == data_mat->c,
+               "slope must have size 1 or input.channels");
+}
+
+void PRelu::forward_impl() const {
+    dab_check(dab_prelu_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->n * data_mat->h * data_mat->w,
+                                data_mat->c, static_cast<const float *>(slope_mat->data), (int)slope_mat->total(), stream()));
+}
+
+// dabnn/layers/Concat.cpp:7-21 (two inputs, channel axis)
+Concat::Concat(NetCP net, css name, css input1, css input2, css output)
+    : Layer(net, name, "Concat"), input1_mat(mat(input1)), input2_mat(mat(input2)), output_mat(mat(output)) {
+    BNN_ASSERT(input1_mat->n == input2_mat->n && input1_mat->h == input2_mat->h && input1_mat->w == input2_mat->w,
+               "Wrong input for concat");
+    BNN_ASSERT(output_mat->c == input1_mat->c + input2_mat->c, "Concat output does not hold both inputs");
+}
+
+void Concat::forward_impl() const {
+    dab_check(dab_concat_channels(static_cast<const float *>(input1_mat->data), input1_mat->c,
+                                  static_cast<const float *>(input2_mat->data), input2_mat->c,
+                                  (int64_t)input1_mat->n * input1_mat->h * input1_mat->w,
+                                  static_cast<float *>(output_mat->data), stream()));
+}
+
 // ---------------------------------------------------------------- pooling
 AvePool::AvePool(NetCP net, css name, css input, css output, int kernel_h_, int kernel_w_, int pad_h_, int pad_w_,
                  int stride_h_, int stride_w_)

@@ -1,5 +1,6 @@
-// The layers of the Bi-Real path (dabnn/layers/{BinConv,FloatConv,Affine,Add,
-// AvePool,MaxPool,Relu}.{h,cpp}); constructor signatures follow the reference.
+// The layers of the Bi-Real and BiDenseNet paths (dabnn/layers/{BinConv,FloatConv,
+// Affine,Add,AvePool,MaxPool,Relu,PRelu,Concat}.{h,cpp}); constructor signatures
+// follow the reference.
 #pragma once
 
 #include "layer.h"
@@ -73,6 +74,20 @@ class Relu : public Layer {
    public:
     MatP data_mat;
     Relu(NetCP net, css name, css data);
+    void forward_impl() const override;
+};
+
+class PRelu : public Layer {
+   public:
+    MatP data_mat, slope_mat;
+    PRelu(NetCP net, css name, css data, css slope);
+    void forward_impl() const override;
+};
+
+class Concat : public Layer {
+   public:
+    MatP input1_mat, input2_mat, output_mat;
+    Concat(NetCP net, css name, css input1, css input2, css output);
     void forward_impl() const override;
 };
 

@@ -27,7 +27,7 @@ enum LayerSlot {
     L_CONCAT = 9, L_AFFINE = 10, L_BINARIZE = 11, L_SPLIT = 12, L_SHUFFLE = 13, L_NAME = 14, L_PRELU = 15
 };
 enum LayerType {
-    FpConv2D = 0, AvePoolT, MaxPoolT, ReluT, Softmax, FC, AddT, Concat, BinConv2D, AffineT, Binarize, Split, Shuffle, PRelu
+    FpConv2D = 0, AvePoolT, MaxPoolT, ReluT, Softmax, FC, AddT, ConcatT, BinConv2D, AffineT, Binarize, Split, Shuffle, PReluT
 };
 const char *kLayerTypeNames[] = {"FpConv2D", "AvePool", "MaxPool", "Relu",     "Softmax", "FC",      "Add",
                                  "Concat",   "BinConv2D", "Affine", "Binarize", "Split",   "Shuffle", "PRelu"};
@@ -272,9 +272,30 @@ void Net::prepare(const void *buf) {
                                                                strides[0], strides[1]));
                 break;
             }
+            case PReluT: {
+                const fb::Table p = layer.table(L_PRELU);
+                BNN_ASSERT(p.valid(), "PRelu layer without parameters");
+                const std::string input = p.str(0), slope = p.str(1), output = p.str(2);
+                alias_output(output, input);
+                layers.push_back(std::make_shared<PRelu>(get_weak(), name, input, slope));
+                break;
+            }
+            case ConcatT: {  // dabnn/net.cpp:230-236: two inputs, channel axis; shape as common/Shaper.cpp:157-178
+                const fb::Table p = layer.table(L_CONCAT);
+                BNN_ASSERT(p.valid(), "Concat layer without parameters");
+                BNN_ASSERT(p.scalar<int32_t>(1, 0) == 3, "Concat: axis must be 3");
+                BNN_ASSERT(p.vec_len(0) == 2, "Concat takes two inputs");
+                const std::string in1 = p.vec_str(0, 0), in2 = p.vec_str(0, 1), output = p.str(2);
+                const auto &s1 = shape_of(in1);
+                const auto &s2 = shape_of(in2);
+                BNN_ASSERT(s1[1] == s2[1] && s1[2] == s2[2], "Wrong input for concat");
+                new_output(output, s1[1], s1[2], s1[3] + s2[3]);
+                layers.push_back(std::make_shared<Concat>(get_weak(), name, in1, in2, output));
+                break;
+            }
             default:
                 throw std::runtime_error(std::string("Not supported op ") +
-                                         (type >= 0 && type <= PRelu ? kLayerTypeNames[type] : "unknown"));
+                                         (type >= 0 && type <= PReluT ? kLayerTypeNames[type] : "unknown"));
         }
     }
     if (optimize) fuse_binconv_epilogues();
@@ -298,6 +319,11 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
         writes = {ad->input1_mat.get()};
     } else if (auto re = std::dynamic_pointer_cast<Relu>(l)) {
         reads = writes = {re->data_mat.get()};
+    } else if (auto pr = std::dynamic_pointer_cast<PRelu>(l)) {
+        reads = writes = {pr->data_mat.get()};
+    } else if (auto cc = std::dynamic_pointer_cast<Concat>(l)) {
+        reads = {cc->input1_mat.get(), cc->input2_mat.get()};
+        writes = {cc->output_mat.get()};
     } else if (auto ap = std::dynamic_pointer_cast<AvePool>(l)) {
         reads = {ap->input_mat.get()};
         writes = {ap->output_mat.get()};

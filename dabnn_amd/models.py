@@ -164,3 +164,70 @@ def small_bnn(seed=0, hw=16, width=64):
                    "bias": tensor("fc_bias", (0.1 * r.standard_normal(10)).astype(np.float32)), "output": "logits",
                    "pads": [0] * 4, "strides": [1, 1], "dilations": [1, 1]})
     return layers, inits, [("data", [1, hw, hw, 3])]
+
+
+def dense_bnn(seed=0, hw=16, growth=64):
+    """A BiDenseNet-style miniature (input hw x hw x 3) in the layer vocabulary the converter emits for such nets
+    (tools/onnx2bnn/OnnxConverter.cpp:373-400 PRelu, :490-513 Concat):
+
+      FpConv2D 3x3 (3 -> growth) + Affine + PRelu (one slope per channel)
+      dense block: 3 x [BinConv2D 3x3 (cin -> growth) + Affine, Concat(features, new)]   cin = g, 2g, 3g
+      transition:  MaxPool 2x2 s2, FpConv2D 1x1 (4g -> 2g) + Affine + PRelu (one slope)
+      dense block: 2 x [BinConv2D 3x3 + Affine, Concat]                                   cin = 2g, 3g
+      AvePool (global) + FpConv2D 1x1 with bias (4g -> 10)
+
+    With growth 64 the binary convolutions see 64, 128, 192, 128 and 192 input channels: the direct 3x3 kernel and the
+    im2col + bgemm method with a filter padded to a multiple of 128 bits both run."""
+    r = np.random.default_rng(seed)
+    layers, inits = [], []
+
+    def tensor(name, data, shape=None, align=False):
+        inits.append({"name": name, "shape": list(data.shape if shape is None else shape), "data": data,
+                      "align_hwc_to_128": align})
+        return name
+
+    def fconv(name, src, dst, cin, cout, k, pad, bias=False):
+        w = (r.standard_normal((cout, k, k, cin)) / np.sqrt(k * k * cin)).astype(np.float32)
+        layer = {"type": "FpConv2D", "name": name, "input": src, "weight": tensor(name + "_w", w), "output": dst,
+                 "pads": [pad] * 4, "strides": [1, 1], "dilations": [1, 1]}
+        if bias:
+            layer["bias"] = tensor(name + "_bias", (0.1 * r.standard_normal(cout)).astype(np.float32))
+        layers.append(layer)
+
+    def affine_prelu(p, blob, c, per_channel):
+        a = (1.0 + 0.1 * r.standard_normal(c)).astype(np.float32)
+        b = (0.1 * r.standard_normal(c)).astype(np.float32)
+        layers.append({"type": "Affine", "name": p + "_affine", "input": blob, "a": tensor(p + "_a", a),
+                       "b": tensor(p + "_b", b), "output": blob + "_bn"})
+        slope = r.uniform(0.1, 0.4, c if per_channel else 1).astype(np.float32)
+        layers.append({"type": "PRelu", "name": p + "_prelu", "input": blob + "_bn", "slope": tensor(p + "_slope", slope),
+                       "output": blob + "_act"})
+        return blob + "_act"
+
+    def dense_layer(p, cur, cin):
+        wf = r.standard_normal((growth, 3, 3, cin)).astype(np.float32)
+        wname = tensor(p + "_w", pack_weight(wf).ravel(), shape=[growth, 3, 3, cin], align=(cin != 64))
+        layers.append({"type": "BinConv2D", "name": p + "_bconv", "input": cur, "weight": wname, "output": p + "_cnt",
+                       "pads": [1] * 4, "strides": [1, 1], "dilations": [1, 1]})
+        a, b = fold_bn(np.full(growth, 0.5, np.float32), (0.1 * r.standard_normal(growth)).astype(np.float32),
+                       np.zeros(growth, np.float32), np.full(growth, 9.0 * cin, np.float32), 1e-5, 9 * cin)
+        layers.append({"type": "Affine", "name": p + "_affine", "input": p + "_cnt", "a": tensor(p + "_a", a),
+                       "b": tensor(p + "_b", b), "output": p + "_bn"})
+        layers.append({"type": "Concat", "name": p + "_concat", "inputs": [cur, p + "_bn"], "axis": 3,
+                       "output": p + "_cat"})
+        return p + "_cat", cin + growth
+
+    fconv("conv1", "data", "conv1_out", 3, growth, 3, 1)
+    cur, cin = affine_prelu("stem", "conv1_out", growth, True), growth
+    for i in range(3):
+        cur, cin = dense_layer("d1l%d" % i, cur, cin)
+    layers.append({"type": "MaxPool", "name": "t1_pool", "input": cur, "output": "t1_pool_out", "kernel_shape": [2, 2],
+                   "pads": [0] * 4, "strides": [2, 2]})
+    fconv("t1_conv", "t1_pool_out", "t1_conv_out", cin, cin // 2, 1, 0)
+    cur, cin = affine_prelu("t1", "t1_conv_out", cin // 2, False), cin // 2
+    for i in range(2):
+        cur, cin = dense_layer("d2l%d" % i, cur, cin)
+    layers.append({"type": "AvePool", "name": "gap", "input": cur, "output": "gap_out",
+                   "kernel_shape": [hw // 2, hw // 2], "pads": [0] * 4, "strides": [1, 1]})
+    fconv("fc", "gap_out", "logits", cin, 10, 1, 0, bias=True)
+    return layers, inits, [("data", [1, hw, hw, 3])]

@@ -261,6 +261,34 @@ def add_inplace(a, b):
     return a
 
 
+def relu_inplace(x):
+    """Relu::forward_impl (dabnn/layers/Relu.cpp)."""
+    _need(x, torch.float32, "x")
+    check(lib.dab_relu_inplace(_ptr(x), x.numel(), _stream()))
+    return x
+
+
+def prelu_inplace(x, slope):
+    """PRelu::forward_impl (dabnn/layers/PRelu.cpp:6-30): slope holds one value or one per channel."""
+    _need(x, torch.float32, "x")
+    _need(slope, torch.float32, "slope")
+    c = x.shape[-1]
+    check(lib.dab_prelu_inplace(_ptr(x), x.numel() // c, c, _ptr(slope), slope.numel(), _stream()))
+    return x
+
+
+def concat(a, b):
+    """Concat::forward_impl (dabnn/layers/Concat.cpp:7-21): two NHWC tensors joined along the channel axis."""
+    _need(a, torch.float32, "a")
+    _need(b, torch.float32, "b")
+    if a.shape[:-1] != b.shape[:-1]:
+        raise capi.DabError(capi.DAB_EINVAL, "concat: shapes differ outside the channel axis")
+    ca, cb = a.shape[-1], b.shape[-1]
+    out = _empty(tuple(a.shape[:-1]) + (ca + cb,), torch.float32, a.device)
+    check(lib.dab_concat_channels(_ptr(a), ca, _ptr(b), cb, a.numel() // ca, _ptr(out), _stream()))
+    return out
+
+
 def _pool(fn, x, kh, kw, pad_h, pad_w, stride_h, stride_w):
     _need(x, torch.float32, "x")
     n, h, w, c = x.shape

@@ -183,6 +183,19 @@ DAB_API int dab_add_inplace(float *a, const float *b, int64_t n_elem, dab_stream
 /* Relu::forward_impl (dabnn/layers/Relu.cpp): x = max(x, 0) in place over n_elem floats. */
 DAB_API int dab_relu_inplace(float *x, int64_t n_elem, dab_stream_t stream);
 
+/*
+ * PRelu::forward_impl (dabnn/layers/PRelu.cpp:6-30): x = x < 0 ? x*slope : x in place, with one slope for the whole
+ * tensor (slope_n == 1) or one per channel (slope_n == c); any other slope_n is DAB_EINVAL as the reference asserts.
+ */
+DAB_API int dab_prelu_inplace(float *x, int64_t n_pix, int c, const float *slope, int slope_n, dab_stream_t stream);
+
+/*
+ * Concat::forward_impl (dabnn/layers/Concat.cpp:7-21; axis 3 only, dabnn/net.cpp:230-236): out[p] = a[p][0..ca) followed
+ * by b[p][0..cb) for each of the n_pix pixels.  out must not alias a or b.
+ */
+DAB_API int dab_concat_channels(const float *a, int ca, const float *b, int cb, int64_t n_pix, float *out,
+                                dab_stream_t stream);
+
 /* Mat::fill<float> (dabnn/mat.h:351-443): x[i] = value; the zero-fill before bgemm (dabnn/layers/BinConv.cpp:153). */
 DAB_API int dab_fill_f32(float *x, int64_t n_elem, float value, dab_stream_t stream);
 

@@ -79,6 +79,10 @@ def lib():
         L.orc_affine_inplace.argtypes = [fp, sz, i, fp, fp]
         L.orc_add_inplace.restype = None
         L.orc_add_inplace.argtypes = [fp, fp, sz]
+        L.orc_prelu_inplace.restype = i
+        L.orc_prelu_inplace.argtypes = [fp, sz, i, fp, i]
+        L.orc_concat.restype = None
+        L.orc_concat.argtypes = [fp, i, fp, i, sz, fp]
         L.orc_ave_pool.restype = None
         L.orc_ave_pool.argtypes = [fp, i, i, i, i, i, i, i, i, i, fp]
         L.orc_max_pool.restype = None
@@ -291,6 +295,25 @@ def add_inplace(a, b):
     b, bp = _f(b)
     lib().orc_add_inplace(a.ctypes.data_as(_c_float_p), bp, a.size)
     return a
+
+
+def prelu_inplace(x, slope):
+    assert x.dtype == np.float32 and x.flags["C_CONTIGUOUS"]
+    slope, sp = _f(slope)
+    c = x.shape[-1]
+    if lib().orc_prelu_inplace(x.ctypes.data_as(_c_float_p), x.size // c, c, sp, slope.size) != 0:
+        raise RuntimeError("slope must have size 1 or input.channels")  # dabnn/layers/PRelu.cpp:7-9
+    return x
+
+
+def concat(a, b):
+    a, ap = _f(a)
+    b, bp = _f(b)
+    assert a.shape[:-1] == b.shape[:-1]
+    ca, cb = a.shape[-1], b.shape[-1]
+    out = np.empty(a.shape[:-1] + (ca + cb,), dtype=np.float32)
+    lib().orc_concat(ap, ca, bp, cb, a.size // ca, out.ctypes.data_as(_c_float_p))
+    return out
 
 
 def ave_pool(x, kh, kw, pad_h, pad_w, stride_h, stride_w):

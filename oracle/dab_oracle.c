@@ -30,6 +30,9 @@
  *                                  and with the +-1 float convolution
  *   orc_fconv / pools / affine     torch.nn.functional on NCHW-permuted data;
  *                                  ramp cases of tests/fconv_test.cpp
+ *   orc_prelu_inplace              torch.nn.functional.prelu (scalar and per-
+ *                                  channel slope)
+ *   orc_concat                     numpy.concatenate along the channel axis
  *   orc_pack_weight / orc_bn_fold  K - 2*cnt end-to-end identity
  */
 #include <stddef.h>
@@ -424,6 +427,31 @@ ORC_API void orc_affine_inplace(float *x, size_t n_pix, int c, const float *a, c
 /* dabnn/layers/Add.cpp:7-17: a += b. */
 ORC_API void orc_add_inplace(float *a, const float *b, size_t n) {
     for (size_t i = 0; i < n; ++i) a[i] += b[i];
+}
+
+/*
+ * dabnn/layers/PRelu.cpp:6-30: a negative value is multiplied by the slope
+ * (slope_n == 1) or by its channel's slope (slope_n == c).  Returns nonzero
+ * for any other slope_n, where the reference asserts.
+ */
+ORC_API int orc_prelu_inplace(float *x, size_t n_pix, int c, const float *slope, int slope_n) {
+    if (slope_n != 1 && slope_n != c) return 1;
+    for (size_t p = 0; p < n_pix; ++p)
+        for (int i = 0; i < c; ++i) {
+            float *v = x + p * c + i;
+            if (*v < 0) *v = *v * slope[slope_n == 1 ? 0 : i];
+        }
+    return 0;
+}
+
+/* dabnn/layers/Concat.cpp:7-21: per pixel, the ca values of a and then the cb values of b. */
+ORC_API void orc_concat(const float *a, int ca, const float *b, int cb, size_t n_pix, float *out) {
+    for (size_t p = 0; p < n_pix; ++p) {
+        memcpy(out, a + p * ca, (size_t)ca * sizeof(float));
+        out += ca;
+        memcpy(out, b + p * cb, (size_t)cb * sizeof(float));
+        out += cb;
+    }
 }
 
 /*

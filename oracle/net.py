@@ -3,7 +3,7 @@ top of the oracle kernels.  Test infrastructure only.
 
 Takes the plain model description used by ``dabnn_amd.dab_format`` (layers,
 initializers, inputs) and one NHWC image; returns every blob by name.  Affine,
-Add and Relu work in place and their output name aliases the input blob, as
+Add, Relu and PRelu work in place and their output name aliases the input blob, as
 ADD_INPLACE_LAYER does (common/flatbuffers_helper.h:68-73); BinConv follows
 the x86 dispatch (dabnn/layers/BinConv.cpp:80-98) via orc.binconv_forward.
 """
@@ -49,6 +49,13 @@ def _apply(layer, act, blobs, record=None):
         buf = act[layer["input"]]
         np.maximum(buf, 0, out=buf)
         act[layer["output"]] = buf
+    elif ty == "PRelu":
+        buf = act[layer["input"]]
+        orc.prelu_inplace(buf, np.asarray(blobs[layer["slope"]]["data"]))
+        act[layer["output"]] = buf
+    elif ty == "Concat":
+        assert layer["axis"] == 3 and len(layer["inputs"]) == 2  # dabnn/net.cpp:230-236
+        act[layer["output"]] = orc.concat(act[layer["inputs"][0]], act[layer["inputs"][1]])
     elif ty in ("MaxPool", "AvePool"):
         src = act[layer["input"]]
         kh, kw = layer["kernel_shape"]
@@ -68,7 +75,7 @@ def run_model(layers, initializers, x, record=None):
     return act
 
 
-_INPLACE = {"Affine": "input", "Add": "input1", "Relu": "input"}
+_INPLACE = {"Affine": "input", "Add": "input1", "Relu": "input", "PRelu": "input"}
 
 
 def run_segments(layers, initializers, fetch):
@@ -102,9 +109,8 @@ def run_segments(layers, initializers, fetch):
     for seg in segs:
         act = {}
         first = seg[0]
-        for key in ("input", "input1", "input2"):
-            if key in first:
-                act[first[key]] = np.array(fetch(r(first[key])), dtype=np.float32, copy=True)
+        for name in [first[key] for key in ("input", "input1", "input2") if key in first] + list(first.get("inputs", [])):
+            act[name] = np.array(fetch(r(name)), dtype=np.float32, copy=True)
         for layer in seg:
             if layer is not first and layer["type"] == "Add":
                 act[layer["input2"]] = np.array(fetch(r(layer["input2"])), dtype=np.float32, copy=True)

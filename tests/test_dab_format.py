@@ -23,6 +23,18 @@ def test_roundtrip_bireal18():
         assert sum(l["type"] == "BinConv2D" for l in layers) == 16
 
 
+def test_roundtrip_dense_net_with_concat_and_prelu():
+    layers, inits, inputs = models.dense_bnn(4)
+    m = df.read_model(df.write_model(layers, inits, inputs))
+    assert [l["type"] for l in m["layers"]].count("Concat") == 5 and [l["type"] for l in m["layers"]].count("PRelu") == 2
+    for a, b in zip(layers, m["layers"]):
+        for k, v in a.items():
+            assert b[k] == v, (a["name"], k)
+    for a, b in zip(inits, m["initializers"]):
+        assert (a["name"], a["shape"]) == (b["name"], b["shape"])
+        assert np.array_equal(np.asarray(a["data"]).ravel(), b["data"])
+
+
 def test_layout_rules():
     layers, inits, inputs = models.small_bnn(0)
     buf = df.write_model(layers, inits, inputs)

@@ -379,6 +379,31 @@ def test_affine_add_bit_exact(dab):
     np.testing.assert_array_equal(got2, want + y)
 
 
+@pytest.mark.parametrize("shape", [(2, 5, 7, 64), (1, 3, 3, 5), (3, 16, 16, 192), (1, 1, 1, 1)])
+def test_prelu_bit_exact(dab, shape):
+    r = rng(44)
+    x = r.standard_normal(shape).astype(np.float32)
+    x.ravel()[:2] = [0.0, -0.0][:x.size]
+    for slope in (np.array([0.25], np.float32), r.uniform(-0.5, 0.5, shape[-1]).astype(np.float32)):
+        got = dab.prelu_inplace(dev_f(x), dev_f(slope)).cpu().numpy()
+        want = np.stack([orc.prelu_inplace(img.copy(), slope) for img in x])
+        np.testing.assert_array_equal(got, want)
+    if shape[-1] > 2:
+        with pytest.raises(RuntimeError, match="slope must have size 1 or c"):
+            dab.prelu_inplace(dev_f(x), dev_f(np.ones(2, np.float32)))
+
+
+@pytest.mark.parametrize("n,h,w,ca,cb", [(2, 5, 7, 64, 64), (1, 3, 3, 5, 2), (3, 16, 16, 128, 64), (1, 1, 1, 1, 1)])
+def test_concat_bit_exact(dab, n, h, w, ca, cb):
+    r = rng(45)
+    a = r.standard_normal((n, h, w, ca)).astype(np.float32)
+    b = r.standard_normal((n, h, w, cb)).astype(np.float32)
+    got = dab.concat(dev_f(a), dev_f(b)).cpu().numpy()
+    np.testing.assert_array_equal(got, np.stack([orc.concat(x, y) for x, y in zip(a, b)]))
+    with pytest.raises(RuntimeError, match="shapes differ"):
+        dab.concat(dev_f(a), dev_f(b[:, :, :-1] if w > 1 else np.zeros((n, h, w + 1, cb), np.float32)))
+
+
 @pytest.mark.parametrize("n,h,w,c,k,pad,stride", [(1, 8, 8, 4, 2, 0, 2), (2, 7, 7, 512, 7, 0, 1), (1, 9, 6, 4, 3, 1, 2),
                                                   (1, 112, 112, 64, 3, 1, 2), (2, 56, 56, 64, 2, 0, 2)])
 def test_pools(dab, n, h, w, c, k, pad, stride):

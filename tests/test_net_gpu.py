@@ -33,7 +33,7 @@ def check_every_segment(n, layers, inits, image):
     checked = 0
     for name, first_type, want in orc_net.run_segments(layers, inits, lambda b: n.get_blob(b)[image]):
         got = n.get_blob(name)[image]
-        if first_type in ("BinConv2D", "MaxPool", "Affine", "Add", "Relu"):
+        if first_type in ("BinConv2D", "MaxPool", "Affine", "Add", "Relu", "PRelu", "Concat"):
             np.testing.assert_array_equal(got, want, err_msg=name)
         else:
             close(got, want)
@@ -82,6 +82,27 @@ def test_small_net_matches_cpu_layer_loop(mods):
             packed = n.get_blob("binaized_for_%s_cnt_cal" % blk)[i]
             src = {"b0": "conv1_out", "b1": "b0_out", "b2": "b1_bn"}[blk]
             assert packed.shape == orc.pack_mat(cpu[src]).shape
+    n.close()
+
+
+def test_dense_net_with_concat_and_prelu_matches_cpu_layer_loop(mods):
+    """A BiDenseNet-style graph: Concat joins each binary convolution's result to its input features, PRelu (one slope
+    and one per channel) follows the float convolutions, and the binary convolutions see 64/128/192 channels."""
+    df, models, net = mods
+    layers, inits, inputs = models.dense_bnn(3, hw=16)
+    batch = 2
+    x = np.random.default_rng(9).standard_normal((batch, 16, 16, 3)).astype(np.float32)
+    n = net.Net(batch=batch).read_buf(df.write_model(layers, inits, inputs))
+    descs = n.layers()
+    assert sum(d.startswith("Concat") for d in descs) == 5 and sum(d.startswith("PRelu") for d in descs) == 2
+    assert sum("DIRECT_CONV" in d for d in descs) == 3 and sum("BGEMM" in d for d in descs) == 2
+    n.run(x)
+    logits = n.get_blob("logits").reshape(batch, -1)
+    for i in range(batch):
+        assert check_every_segment(n, layers, inits, i) == 15
+        assert check_packed_inputs(n, layers, i) == 3
+        drift_ok(logits[i], orc_net.run_model(layers, inits, x[i])["logits"])
+    assert n.get_blob("d1l2_cat").shape == (batch, 16, 16, 256)
     n.close()
 
 
@@ -167,6 +188,9 @@ def test_error_paths(mods, tmp_path):
     bad = layers + [{"type": "Softmax", "name": "sm", "input": "logits", "output": "prob"}]
     with pytest.raises(RuntimeError, match="Not supported op Softmax"):
         net.Net().read_buf(df.write_model(bad, inits, inputs))
+    shuffle = [{"type": "Shuffle", "name": "sh", "input": "data", "output": "out"}]
+    with pytest.raises(RuntimeError, match="Not supported op Shuffle"):
+        net.Net().read_buf(df.write_model(shuffle, [], [("data", [1, 4, 4, 128])]))
     n = net.Net().read_buf(df.write_model(layers, inits, inputs))
     with pytest.raises(KeyError):
         n.get_blob("no_such_blob")

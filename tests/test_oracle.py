@@ -357,6 +357,22 @@ def test_affine_and_add():
     np.testing.assert_array_equal(orc.add_inplace(x.copy(), y), x + y)
 
 
+def test_prelu_vs_torch_and_concat_vs_numpy():
+    """dabnn/layers/PRelu.cpp:6-30 against torch.nn.functional.prelu (NCHW, so the slope indexes dim 1) for one slope
+    and for one slope per channel; dabnn/layers/Concat.cpp:7-21 against numpy.concatenate on the channel axis."""
+    x = rng(48).standard_normal((5, 4, 8)).astype(np.float32)
+    x[0, 0, :3] = [0.0, -0.0, -1.0]
+    xt = torch.from_numpy(x).permute(2, 0, 1)[None]
+    for slope in (np.array([0.25], np.float32), rng(49).uniform(-0.5, 0.5, 8).astype(np.float32)):
+        want = F.prelu(xt, torch.from_numpy(slope))[0].permute(1, 2, 0).numpy()
+        np.testing.assert_array_equal(orc.prelu_inplace(x.copy(), slope), want)
+    with pytest.raises(RuntimeError, match="slope must have size 1 or input.channels"):
+        orc.prelu_inplace(x.copy(), np.ones(3, np.float32))
+    y = rng(50).standard_normal((5, 4, 3)).astype(np.float32)
+    np.testing.assert_array_equal(orc.concat(x, y), np.concatenate([x, y], axis=-1))
+    np.testing.assert_array_equal(orc.concat(y, x), np.concatenate([y, x], axis=-1))
+
+
 @pytest.mark.parametrize("h,w,c,k,pad,stride", [(8, 8, 4, 2, 0, 2), (7, 7, 8, 7, 0, 1), (9, 6, 4, 3, 1, 2),
                                                 (112, 112, 4, 3, 1, 2)])
 def test_pools_vs_torch(h, w, c, k, pad, stride):
