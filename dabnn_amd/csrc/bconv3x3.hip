@@ -10,6 +10,8 @@
 // resident; out-of-image taps are fetched through a buffer descriptor with an
 // out-of-range offset, which the hardware answers with zero -- the zero word
 // that stands for 64 values of -1 (dabnn/pad.h:12).
+#include <type_traits>
+
 #include "xnor_core.h"
 
 namespace dab {
@@ -75,6 +77,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     constexpr int WCH = Residency<CW, NARROW>::window;
     constexpr int WU = WCH / Q;  // units per staging window
     constexpr int kStageBytes = Stage<WCH>::bytes;
+    constexpr int kFlushGroup = CW == 1 ? 8 : CW == 2 ? (NARROW ? 8 : 2) : CW == 4 ? 4 : 1;  // shortcut loads in flight, as the register budget allows
     __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
     const int lane = threadIdx.x & 63;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -93,7 +96,26 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     bool need_load = true;
     uint32_t a[K32];
 
-    for (int u = u0; u < u1; ++u) {
+    auto flush = [&](auto group, int cg_now, int slot) {
+        constexpr int G = decltype(group)::value;
+        if constexpr (MODE == kModeAffineAddSign) {
+            EpiAffineAddSign epi;
+            epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+            epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
+            stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
+                                (slot * Q + Q - 1) >> 2, epi);
+        } else if constexpr (MODE == kModeAffineAdd) {
+            EpiAffineAdd epi;
+            epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+            stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
+                                (slot * Q + Q - 1) >> 2, epi);
+        } else {
+            stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
+                                (slot * Q + Q - 1) >> 2, EpiStore());
+        }
+    };
+
+    for (int u = u0;; ++u) {
         if (need_load) {
             need_load = false;
             int pix = tile * 64 + lane;
@@ -145,23 +167,14 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
         const int slot = cg % WU;
         stage_put<WCH, Q>(stage, lane, slot * Q, acc);
 
+        // The window goes out when it is full or the tile ends.  The last unit of the wave leaves the loop first:
+        // its flush runs where the activation registers are dead, so it can keep all of the window's shortcut loads
+        // in flight at once -- every wave of a launch reaches that flush at about the same time, with no other
+        // wave's arithmetic to hide the memory latency behind.
+        if (u == u1 - 1) break;
         const bool last_in_tile = cg == p.n_groups - 1;
-        if (slot == WU - 1 || last_in_tile || u == u1 - 1) {
-            if constexpr (MODE == kModeAffineAddSign) {
-                EpiAffineAddSign epi;
-                epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
-                epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
-                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
-                                 (slot * Q + Q - 1) >> 2, epi);
-            } else if constexpr (MODE == kModeAffineAdd) {
-                EpiAffineAdd epi;
-                epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
-                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
-                                 (slot * Q + Q - 1) >> 2, epi);
-            } else {
-                stage_flush<WCH>(stage, lane, p.out, p.cout, tile, p.total, (cg - slot) * Q, ch_lo >> 2,
-                                 (slot * Q + Q - 1) >> 2, EpiStore());
-            }
+        if (slot == WU - 1 || last_in_tile) {
+            flush(std::integral_constant<int, kFlushGroup>{}, cg, slot);
             ch_lo = 0;
         }
         if (last_in_tile) {
@@ -172,6 +185,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             ++cg;
         }
     }
+    flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
 template <int CW, int MODE, bool NARROW>

@@ -209,11 +209,17 @@ __device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch
 //                     (pack_mat, dabnn/bitpack.h:277-293)
 struct EpiStore {
     static constexpr bool kEmit = false;
+    static constexpr bool kShortcut = false;  // the epilogue never reads a second tensor
+    const float *shortcut = nullptr;
     __device__ __forceinline__ void prepare(int) {}
-    __device__ __forceinline__ float4 operator()(float4 v, const float4 *, size_t) const { return v; }
+    template <bool SC>
+    __device__ __forceinline__ float4 apply(float4 v, float4) const {
+        return v;
+    }
 };
 struct EpiAffineAdd {
     static constexpr bool kEmit = false;
+    static constexpr bool kShortcut = true;
     const float *a;
     const float *b;
     const float *shortcut;  // may be null; same layout as out
@@ -222,15 +228,13 @@ struct EpiAffineAdd {
         av = *reinterpret_cast<const float4 *>(a + ch);
         bv = *reinterpret_cast<const float4 *>(b + ch);
     }
-    __device__ __forceinline__ float4 operator()(float4 v, const float4 *, size_t off) const {
+    template <bool SC>
+    __device__ __forceinline__ float4 apply(float4 v, float4 sc) const {
 #pragma clang fp contract(off)
         float4 r;
         r.x = av.x * v.x, r.y = av.y * v.y, r.z = av.z * v.z, r.w = av.w * v.w;
         r.x = r.x + bv.x, r.y = r.y + bv.y, r.z = r.z + bv.z, r.w = r.w + bv.w;
-        if (shortcut) {
-            const float4 sc = *reinterpret_cast<const float4 *>(shortcut + off);
-            r.x = r.x + sc.x, r.y = r.y + sc.y, r.z = r.z + sc.z, r.w = r.w + sc.w;
-        }
+        if constexpr (SC) r.x = r.x + sc.x, r.y = r.y + sc.y, r.z = r.z + sc.z, r.w = r.w + sc.w;
         return r;
     }
 };
@@ -240,32 +244,39 @@ struct EpiAffineAddSign : EpiAffineAdd {
     int bits_ld;          // cout / 8
 };
 
-
-// Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
-// WCH-channel window that starts at channel cbase.  out is [pixel][ld] floats;
-// pixels >= total are skipped.
-template <int WCH, class Epi>
-__device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
-                                            int tile, int total, int cbase, int p_lo, int p_hi, Epi epi) {
-    __builtin_amdgcn_wave_barrier();
-    const int np = p_hi - p_lo + 1;  // 16-byte parts per pixel row
+// The whole-window store pass of stage_flush: lane = (pixel row pr0, 16-byte part), NP store instructions of
+// 64/NP pixels each.  The shortcut values of G stores are fetched together before the first of them is used, so a
+// flush waits for memory NP/G times and not once per store (the loads of one store cannot move above the previous
+// store by themselves: the compiler has to assume the two tensors overlap).
+template <int WCH, int G, bool SC, class Epi>
+__device__ __forceinline__ void stage_flush_window(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
+                                                   int tile, int cbase, Epi &epi) {
     constexpr int NP = Stage<WCH>::parts, ROW = Stage<WCH>::row, PPI = 64 / NP;  // PPI pixels per store instruction
-    if (np == NP && (tile + 1) * 64 <= total) {
-        const int pr0 = lane / NP, part = lane % NP;
-        const unsigned char *src = stage + pr0 * ROW + part * 16;
-        const size_t off0 = ((size_t)tile * 64 + pr0) * ld + cbase + part * 4;
-        epi.prepare(cbase + part * 4);
+    static_assert(NP % G == 0, "group size must divide the number of stores");
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    const int pr0 = lane / NP, part = lane % NP;
+    const unsigned char *src = stage + pr0 * ROW + part * 16;
+    const size_t off0 = ((size_t)tile * 64 + pr0) * ld + cbase + part * 4;
+    epi.prepare(cbase + part * 4);
 #pragma unroll
-        for (int i = 0; i < NP; ++i) {
+    for (int i0 = 0; i0 < NP; i0 += G) {
+        float4 sc[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if constexpr (SC)
+                sc[g] = *reinterpret_cast<const float4 *>(epi.shortcut + off0 + (size_t)(i0 + g) * PPI * ld);
+            else
+                sc[g] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int i = i0 + g;
             const float4 v = *reinterpret_cast<const float4 *>(src + i * PPI * ROW);
-            const size_t off = off0 + (size_t)i * PPI * ld;
-            float4 *d = reinterpret_cast<float4 *>(out + off);
+            const float4 r = epi.template apply<SC>(v, sc[g]);
+            const f32x4 rv = {r.x, r.y, r.z, r.w};
             // streaming store: the output is not read again by this kernel, and lines that leave the L2 early do
             // not have to be written back when the kernel ends
-            typedef float f32x4 __attribute__((ext_vector_type(4)));
-            const float4 r = epi(v, d, off);
-            const f32x4 rv = {r.x, r.y, r.z, r.w};
-            __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(d));
+            __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(out + off0 + (size_t)i * PPI * ld));
             if constexpr (Epi::kEmit) {
                 // the NP lanes of a pixel hold its window's sign bits, four each: gather them in the first lane
                 uint32_t w = sign_nibble(r) << (4 * part);
@@ -281,6 +292,25 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
                 }
             }
         }
+    }
+}
+
+// Writes the staged 16-byte parts [p_lo, p_hi] (4 channels each) of the
+// WCH-channel window that starts at channel cbase.  out is [pixel][ld] floats;
+// pixels >= total are skipped.  G: shortcut loads kept in flight in the whole-window pass.
+template <int WCH, int G, class Epi>
+__device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
+                                            int tile, int total, int cbase, int p_lo, int p_hi, Epi epi) {
+    __builtin_amdgcn_wave_barrier();
+    const int np = p_hi - p_lo + 1;  // 16-byte parts per pixel row
+    constexpr int NP = Stage<WCH>::parts, ROW = Stage<WCH>::row;
+    constexpr int GG = G < NP ? G : NP;
+    const bool has_sc = Epi::kShortcut && epi.shortcut != nullptr;
+    if (np == NP && (tile + 1) * 64 <= total) {
+        if (has_sc)
+            stage_flush_window<WCH, GG, Epi::kShortcut>(stage, lane, out, ld, tile, cbase, epi);
+        else
+            stage_flush_window<WCH, GG, false>(stage, lane, out, ld, tile, cbase, epi);
     } else {
         const int magic = (65536 + np - 1) / np;  // c / np for c < 512
         for (int i = 0; i < np; ++i) {
@@ -292,10 +322,13 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
             if (pix < total) {
                 const float4 v = *reinterpret_cast<const float4 *>(stage + pr * ROW + part * 16);
                 const size_t off = (size_t)pix * ld + cbase + part * 4;
-                float4 *d = reinterpret_cast<float4 *>(out + off);
                 epi.prepare(cbase + part * 4);
-                const float4 r = epi(v, d, off);
-                *d = r;
+                float4 r;
+                if (has_sc)
+                    r = epi.template apply<Epi::kShortcut>(v, *reinterpret_cast<const float4 *>(epi.shortcut + off));
+                else
+                    r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
+                *reinterpret_cast<float4 *>(out + off) = r;
                 if constexpr (Epi::kEmit) nib = sign_nibble(r);
             }
             if constexpr (Epi::kEmit) {
