@@ -366,7 +366,7 @@ struct PoolVecArgs {
 
 // SIGN (c % 64 == 0): the 16 threads that hold the 64 channels of a word are one row of lanes; their sign nibbles are
 // gathered with DPP and the first of them stores pack_mat's word of the pooled pixel (dabnn/bitpack.h:277-293).
-template <bool MAX, bool SIGN>
+template <bool MAX, bool SIGN, int U>
 __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict__ x, float4 *__restrict__ out,
                                                         uint64_t *__restrict__ out_packed, const PoolVecArgs p) {
     const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
@@ -379,21 +379,31 @@ __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict
     const int oy = (int)(t2 - img * p.g.oh);
     float4 m = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX), sum = make_float4(0.f, 0.f, 0.f, 0.f);
     const int ys = oy * p.g.stride_h - p.g.pad_h, xs = ox * p.g.stride_w - p.g.pad_w;
-    // in-bounds part of the window, so that the tap loop has no branches and its loads overlap
+    // in-bounds part of the window: the taps are walked in the reference's order, U loads at a time, all of them in
+    // flight before the first is used (a 7x7 window is five waits for memory, not 49)
     const int a_lo = ys < 0 ? -ys : 0, a_hi = ys + p.g.kh > p.g.h ? p.g.h - ys : p.g.kh;
     const int b_lo = xs < 0 ? -xs : 0, b_hi = xs + p.g.kw > p.g.w ? p.g.w - xs : p.g.kw;
     const int cnt = (a_hi > a_lo && b_hi > b_lo) ? (a_hi - a_lo) * (b_hi - b_lo) : 0;
-    for (int a = a_lo; a < a_hi; ++a) {
-        const float4 *row = x + (((size_t)img * p.g.h + ys + a) * p.g.w + xs) * p.c4 + ch;
-#pragma unroll 8
-        for (int b = b_lo; b < b_hi; ++b) {
-            const float4 v = row[(size_t)b * p.c4];
-            if (MAX) {
-                m.x = v.x > m.x ? v.x : m.x, m.y = v.y > m.y ? v.y : m.y;
-                m.z = v.z > m.z ? v.z : m.z, m.w = v.w > m.w ? v.w : m.w;
-            } else {
+    const float4 *img0 = x + (size_t)img * p.g.h * p.g.w * p.c4 + ch;
+    int a = a_lo, b = b_lo;
+    for (int t0 = 0; t0 < cnt; t0 += U) {
+        float4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            // past the last tap (a, b) stays on it: a load of a valid address whose value is not used
+            v[u] = img0[((size_t)(ys + a) * p.g.w + (xs + b)) * p.c4];
+            if (t0 + u + 1 < cnt && ++b == b_hi) b = b_lo, ++a;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (t0 + u < cnt) {
+                if (MAX) {
+                    m.x = v[u].x > m.x ? v[u].x : m.x, m.y = v[u].y > m.y ? v[u].y : m.y;
+                    m.z = v[u].z > m.z ? v[u].z : m.z, m.w = v[u].w > m.w ? v[u].w : m.w;
+                } else {
 #pragma clang fp contract(off)
-                sum.x = sum.x + v.x, sum.y = sum.y + v.y, sum.z = sum.z + v.z, sum.w = sum.w + v.w;
+                    sum.x = sum.x + v[u].x, sum.y = sum.y + v[u].y, sum.z = sum.z + v[u].z, sum.w = sum.w + v[u].w;
+                }
             }
         }
     }
@@ -591,12 +601,19 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
         const unsigned vb = (v.total + 255u) / 256u;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         float4 *o4 = reinterpret_cast<float4 *>(out);
+        const int taps = kh * kw;  // loads kept in flight: the whole window up to 3x3, 16 at a time beyond
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, out_packed, v);
+        };
         if (want_sign)
-            hipLaunchKernelGGL((pool_vec4_kernel<true, true>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, out_packed, v);
+            taps <= 4 ? launch(pool_vec4_kernel<true, true, 4>) : taps <= 9 ? launch(pool_vec4_kernel<true, true, 9>)
+                                                                            : launch(pool_vec4_kernel<true, true, 16>);
         else if (is_max)
-            hipLaunchKernelGGL((pool_vec4_kernel<true, false>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, nullptr, v);
+            taps <= 4 ? launch(pool_vec4_kernel<true, false, 4>) : taps <= 9 ? launch(pool_vec4_kernel<true, false, 9>)
+                                                                             : launch(pool_vec4_kernel<true, false, 16>);
         else
-            hipLaunchKernelGGL((pool_vec4_kernel<false, false>), dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, nullptr, v);
+            taps <= 4 ? launch(pool_vec4_kernel<false, false, 4>) : taps <= 9 ? launch(pool_vec4_kernel<false, false, 9>)
+                                                                              : launch(pool_vec4_kernel<false, false, 16>);
         DAB_LAUNCH_CHECK();
         return DAB_OK;
     }
