@@ -28,6 +28,10 @@ namespace dab {
 // with one 16-byte LDS read and uses them in four instructions.
 // Epilogue: + bias, then optionally the Affine (a*v + b, two roundings) and Relu
 // layers that follow the convolution, in the reference's order of operations.
+// CV = 3 is the loader for three-channel images (the 7x7 stem): a lane fetches
+// the three channels of one tap with one 12-byte load, so a slice (8 taps = 24
+// depths) takes a third of the load instructions and of the address and bounds
+// arithmetic per depth.
 struct FconvArgs {
     const float *x;
     const float *w;
@@ -54,17 +58,20 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr uint32_t kOob = 0x80000000u;     // descriptors here are shorter than 2^30 bytes
 constexpr uint32_t kOobRow = 0x40000000u;  // kOobRow + kOob and kOobRow + (anything < 2^30) stay out of range
 
-template <int BM, int BN, int SK, int KSPLIT, bool PADDED>
+template <int BM, int BN, int SK, int KSPLIT, bool PADDED, int CV = 1>
 __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     constexpr int WAVES_MN = 4 / KSPLIT;
     constexpr int WAVES_N = (WAVES_MN >= 2 && BN >= 64) ? 2 : 1, WAVES_M = WAVES_MN / WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;  // wave tile
     constexpr int TM = WTM / 32, TN = WTN / 32;            // 32 x 32 matrix-core tiles per wave
-    constexpr int RP = 256 / SK;                           // tile rows fetched per pass of the block
+    constexpr int LK = SK / CV;                            // loader lanes along the depth (taps when CV == 3)
+    constexpr int RP = 256 / LK;                           // tile rows fetched per pass of the block
     constexpr int APT = BM / RP, BPT = BN / RP;            // loads per thread and slice
     constexpr int RS = SK + 4;                             // LDS row stride: 16-byte reads of 16 lanes hit 64 banks once
+    constexpr int WK = SK / KSPLIT;                        // depths of a slice one wave multiplies
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
-    static_assert(SK == 16 * KSPLIT && APT >= 1 && BPT >= 1, "slice");
+    static_assert(WK % 8 == 0 && 256 % LK == 0 && APT >= 1 && BPT >= 1, "slice");
+    static_assert(CV == 1 || (CV == 3 && KSPLIT == 1), "channel-vector loader");
     __shared__ __attribute__((aligned(16))) float As[2][BM][RS];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RS];
     __shared__ float red[KSPLIT > 1 ? KSPLIT * 16 * 64 : 1];
@@ -82,7 +89,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     const auto o_rsrc = make_rsrc(p.out + (size_t)m0 * p.cout, (uint32_t)rows_m * p.cout * 4u);
 
     // loader: depth l_k of the slice, tile rows l_r + RP*i
-    const int l_k = tid % SK, l_r = tid / SK;
+    const int l_k = tid % LK, l_r = tid / LK;
     uint32_t a_base[APT];  // byte offset of (image, y0, x0, channel 0) from the descriptor's start, modulo 2^32
     int a_y0[PADDED ? APT : 1], a_x0[PADDED ? APT : 1];
     {
@@ -127,11 +134,26 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
 #pragma unroll
     for (int j = 0; j < BPT; ++j) b_row[j] = (uint32_t)(l_r + RP * j) * p.K * 4u;
 
-    float a_reg[APT], b_reg[BPT];
+    typedef float f32xcv __attribute__((ext_vector_type(CV == 3 ? 3 : 1)));
+    f32xcv a_reg[APT], b_reg[BPT];
+    auto load_cv = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off) -> f32xcv {
+        // the result is bit-cast as a whole: casting single elements of a vector buffer load makes the compiler
+        // replace it by one 4-byte load
+        if constexpr (CV == 1)
+            return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0));
+        else
+            return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)off, 0, 0));
+    };
     auto fetch = [&](int k0) {
-        const int k = k0 + l_k;
+        // CV == 1: lane = depth index k -> (tap, channel).  CV == 3: lane = tap, channels 0..2 (c == 3, k0 % 24 == 0).
+        const int k = CV == 1 ? k0 + l_k : k0 + 3 * l_k;
         const bool k_ok = k < p.K;
-        const int tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
+        int tap, ch;
+        if constexpr (CV == 1) {
+            tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
+        } else {
+            tap = (int)((uint32_t)k0 / 3u) + l_k, ch = 0;
+        }
         const int ty = (int)p.div_kw.div((uint32_t)tap), tx = tap - ty * p.kw;
         const int dy = ty * p.dil_h, dx = tx * p.dil_w;
         const uint32_t delta = k_ok ? (uint32_t)((dy * p.wd + dx) * p.c + ch) * 4u : kOob;
@@ -142,18 +164,21 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
                 const int y = a_y0[i] + dy, xx = a_x0[i] + dx;
                 off = ((unsigned)y < (unsigned)p.h && (unsigned)xx < (unsigned)p.wd) ? off : kOob;
             }
-            a_reg[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, (int)off, 0, 0));
+            a_reg[i] = load_cv(x_rsrc, off);
         }
         const uint32_t k4 = k_ok ? (uint32_t)k * 4u : kOob;
 #pragma unroll
-        for (int j = 0; j < BPT; ++j)
-            b_reg[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, (int)(b_row[j] + k4), 0, 0));
+        for (int j = 0; j < BPT; ++j) b_reg[j] = load_cv(w_rsrc, b_row[j] + k4);
     };
     auto commit = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < APT; ++i) As[buf][l_r + RP * i][l_k] = a_reg[i];
+        for (int i = 0; i < APT; ++i)
 #pragma unroll
-        for (int j = 0; j < BPT; ++j) Bs[buf][l_r + RP * j][l_k] = b_reg[j];
+            for (int c = 0; c < CV; ++c) As[buf][l_r + RP * i][l_k * CV + c] = a_reg[i][c];
+#pragma unroll
+        for (int j = 0; j < BPT; ++j)
+#pragma unroll
+            for (int c = 0; c < CV; ++c) Bs[buf][l_r + RP * j][l_k * CV + c] = b_reg[j][c];
     };
 
     f32x16 acc[TM][TN];
@@ -174,8 +199,8 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
         const bool more = k0 + SK < p.K;
         if (more) fetch(k0 + SK);
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {  // this wave's 16 depths of the slice, 8 at a time
-            const int kb = ks * 16 + g * 8 + f_k * 4;
+        for (int g = 0; g < WK / 8; ++g) {  // this wave's depths of the slice, 8 at a time
+            const int kb = ks * WK + g * 8 + f_k * 4;
             float4 a4[TM], b4[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i) a4[i] = *reinterpret_cast<const float4 *>(&As[buf][wm * WTM + i * 32 + f_i][kb]);
@@ -486,9 +511,18 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
         else                                                                                             \
             hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false>), grid, dim3(256), 0, s, a);     \
     } while (0)
+    // three-channel images with a window of enough taps that slices of eight taps waste little (7x7: 56 for 49)
+    const int taps = kh * kw;
+    const bool channel_vectors = c == 3 && bn == 64 && (taps + 7) / 8 * 24 * 10 <= (a.K + 15) / 16 * 16 * 11;
     if (big_tiles < simd_count() / 4) {
         // fewer big tiles than CUs: 32 x 32 tiles, each slice's depth split over the block's waves
         DAB_FCONV_LAUNCH(32, 32, 64, 4);
+    } else if (channel_vectors) {
+        const dim3 grid((unsigned)((M + 127) / 128), (unsigned)((cout + 63) / 64));
+        if (padded)
+            hipLaunchKernelGGL((fconv_kernel<128, 64, 24, 1, true, 3>), grid, dim3(256), 0, s, a);
+        else
+            hipLaunchKernelGGL((fconv_kernel<128, 64, 24, 1, false, 3>), grid, dim3(256), 0, s, a);
     } else if (bn == 32) {
         DAB_FCONV_LAUNCH(128, 32, 16, 1);
     } else if (bn == 64) {
