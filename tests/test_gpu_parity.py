@@ -307,6 +307,10 @@ RTOL = 1e-4
     (1, 32, 3, 64, 7, 3, 2, 1, False), (2, 7, 64, 128, 1, 0, 1, 1, False), (3, 1, 512, 1000, 1, 0, 1, 1, True),
     (1, 17, 5, 70, 3, 1, 2, 1, True), (2, 9, 3, 32, 3, 1, 2, 1, False), (1, 23, 16, 20, 3, 1, 1, 1, True),
     (1, 12, 7, 200, 5, 2, 1, 1, True), (130, 1, 33, 65, 1, 0, 1, 1, False), (1, 40, 8, 8, 3, 1, 1, 1, False),
+    # three-channel images large enough for the big-tile kernels: ragged pixel and channel tiles, with and without
+    # padding, stride 1 and 2, dilation (the 7x7 cases take the one-load-per-tap loader)
+    (5, 180, 3, 40, 7, 3, 2, 1, True), (5, 181, 3, 64, 7, 0, 2, 1, False), (2, 150, 3, 33, 7, 3, 1, 1, False),
+    (4, 200, 3, 64, 7, 6, 2, 2, True), (4, 190, 3, 24, 3, 1, 2, 1, True),
 ])
 def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
     r = rng(40)
