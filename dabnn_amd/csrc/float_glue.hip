@@ -31,7 +31,8 @@ namespace dab {
 // CV = 3 is the loader for three-channel images (the 7x7 stem): a lane fetches
 // the three channels of one tap with one 12-byte load, so a slice (8 taps = 24
 // depths) takes a third of the load instructions and of the address and bounds
-// arithmetic per depth.
+// arithmetic per depth.  CV = 4 does the same with 16-byte loads of four
+// consecutive channels when the channel count is a multiple of 4.
 struct FconvArgs {
     const float *x;
     const float *w;
@@ -66,12 +67,13 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     constexpr int TM = WTM / 32, TN = WTN / 32;            // 32 x 32 matrix-core tiles per wave
     constexpr int LK = SK / CV;                            // loader lanes along the depth (taps when CV == 3)
     constexpr int RP = 256 / LK;                           // tile rows fetched per pass of the block
-    constexpr int APT = BM / RP, BPT = BN / RP;            // loads per thread and slice
+    constexpr int APT = BM / RP, BPT = (BN + RP - 1) / RP;  // loads per thread and slice
     constexpr int RS = SK + 4;                             // LDS row stride: 16-byte reads of 16 lanes hit 64 banks once
     constexpr int WK = SK / KSPLIT;                        // depths of a slice one wave multiplies
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert(WK % 8 == 0 && 256 % LK == 0 && APT >= 1 && BPT >= 1, "slice");
-    static_assert(CV == 1 || (CV == 3 && KSPLIT == 1), "channel-vector loader");
+    static_assert(CV == 1 || CV == 4 || (CV == 3 && KSPLIT == 1), "channel-vector loader");
+    constexpr bool B_PARTIAL = BN < RP;  // fewer weight rows than loader rows: the upper loader rows fetch nothing
     __shared__ __attribute__((aligned(16))) float As[2][BM][RS];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RS];
     __shared__ float red[KSPLIT > 1 ? KSPLIT * 16 * 64 : 1];
@@ -134,22 +136,25 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
 #pragma unroll
     for (int j = 0; j < BPT; ++j) b_row[j] = (uint32_t)(l_r + RP * j) * p.K * 4u;
 
-    typedef float f32xcv __attribute__((ext_vector_type(CV == 3 ? 3 : 1)));
+    typedef float f32xcv __attribute__((ext_vector_type(CV)));
     f32xcv a_reg[APT], b_reg[BPT];
     auto load_cv = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off) -> f32xcv {
         // the result is bit-cast as a whole: casting single elements of a vector buffer load makes the compiler
         // replace it by one 4-byte load
         if constexpr (CV == 1)
             return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0));
-        else
+        else if constexpr (CV == 3)
             return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)off, 0, 0));
+        else
+            return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
     };
     auto fetch = [&](int k0) {
-        // CV == 1: lane = depth index k -> (tap, channel).  CV == 3: lane = tap, channels 0..2 (c == 3, k0 % 24 == 0).
-        const int k = CV == 1 ? k0 + l_k : k0 + 3 * l_k;
+        // CV == 1: lane = depth index k -> (tap, channel).  CV == 4: four consecutive channels of a tap (c % 4 == 0).
+        // CV == 3: lane = tap, channels 0..2 (c == 3, k0 % 24 == 0).
+        const int k = k0 + CV * l_k;
         const bool k_ok = k < p.K;
         int tap, ch;
-        if constexpr (CV == 1) {
+        if constexpr (CV != 3) {
             tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
         } else {
             tap = (int)((uint32_t)k0 / 3u) + l_k, ch = 0;
@@ -168,17 +173,19 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
         }
         const uint32_t k4 = k_ok ? (uint32_t)k * 4u : kOob;
 #pragma unroll
-        for (int j = 0; j < BPT; ++j) b_reg[j] = load_cv(w_rsrc, b_row[j] + k4);
+        for (int j = 0; j < BPT; ++j) b_reg[j] = load_cv(w_rsrc, (!B_PARTIAL || l_r < BN) ? b_row[j] + k4 : kOob);
     };
     auto commit = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < APT; ++i)
 #pragma unroll
             for (int c = 0; c < CV; ++c) As[buf][l_r + RP * i][l_k * CV + c] = a_reg[i][c];
+        if (!B_PARTIAL || l_r < BN) {
 #pragma unroll
-        for (int j = 0; j < BPT; ++j)
+            for (int j = 0; j < BPT; ++j)
 #pragma unroll
-            for (int c = 0; c < CV; ++c) Bs[buf][l_r + RP * j][l_k * CV + c] = b_reg[j][c];
+                for (int c = 0; c < CV; ++c) Bs[buf][l_r + RP * j][l_k * CV + c] = b_reg[j][c];
+        }
     };
 
     f32x16 acc[TM][TN];
@@ -503,32 +510,43 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
                         (a.ow - 1) * stride_w + (kw - 1) * dil_w >= w;
     const int bn = cout <= 32 ? 32 : cout <= 64 ? 64 : 128;
     const long long big_tiles = ((M + 127) / 128) * ((cout + bn - 1) / bn);
-#define DAB_FCONV_LAUNCH(BM, BN, SK, KSPLIT)                                                             \
+#define DAB_FCONV_LAUNCH(BM, BN, SK, KSPLIT, CV)                                                         \
     do {                                                                                                 \
         const dim3 grid((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN));                \
         if (padded)                                                                                      \
-            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, true>), grid, dim3(256), 0, s, a);      \
+            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, true, CV>), grid, dim3(256), 0, s, a);  \
         else                                                                                             \
-            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false>), grid, dim3(256), 0, s, a);     \
+            hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false, CV>), grid, dim3(256), 0, s, a); \
     } while (0)
-    // three-channel images with a window of enough taps that slices of eight taps waste little (7x7: 56 for 49)
+    // Loader: 16-byte loads of four channels when the channel count allows it; for three-channel images one 12-byte
+    // load per tap if the window has enough taps that slices of eight taps waste little (7x7: 56 for 49); else
+    // element by element.
     const int taps = kh * kw;
-    const bool channel_vectors = c == 3 && bn == 64 && (taps + 7) / 8 * 24 * 10 <= (a.K + 15) / 16 * 16 * 11;
+    const bool vec4 = c % 4 == 0 && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt)) % 16 == 0;
+    const bool vec3 = c == 3 && bn == 64 && (taps + 7) / 8 * 24 * 10 <= (a.K + 15) / 16 * 16 * 11;
     if (big_tiles < simd_count() / 4) {
         // fewer big tiles than CUs: 32 x 32 tiles, each slice's depth split over the block's waves
-        DAB_FCONV_LAUNCH(32, 32, 64, 4);
-    } else if (channel_vectors) {
-        const dim3 grid((unsigned)((M + 127) / 128), (unsigned)((cout + 63) / 64));
-        if (padded)
-            hipLaunchKernelGGL((fconv_kernel<128, 64, 24, 1, true, 3>), grid, dim3(256), 0, s, a);
+        if (vec4)
+            DAB_FCONV_LAUNCH(32, 32, 64, 4, 4);
         else
-            hipLaunchKernelGGL((fconv_kernel<128, 64, 24, 1, false, 3>), grid, dim3(256), 0, s, a);
+            DAB_FCONV_LAUNCH(32, 32, 64, 4, 1);
+    } else if (vec3) {
+        DAB_FCONV_LAUNCH(128, 64, 24, 1, 3);
     } else if (bn == 32) {
-        DAB_FCONV_LAUNCH(128, 32, 16, 1);
+        if (vec4)
+            DAB_FCONV_LAUNCH(128, 32, 16, 1, 4);
+        else
+            DAB_FCONV_LAUNCH(128, 32, 16, 1, 1);
     } else if (bn == 64) {
-        DAB_FCONV_LAUNCH(128, 64, 16, 1);
+        if (vec4)
+            DAB_FCONV_LAUNCH(128, 64, 16, 1, 4);
+        else
+            DAB_FCONV_LAUNCH(128, 64, 16, 1, 1);
     } else {
-        DAB_FCONV_LAUNCH(128, 128, 16, 1);
+        if (vec4)
+            DAB_FCONV_LAUNCH(128, 128, 16, 1, 4);
+        else
+            DAB_FCONV_LAUNCH(128, 128, 16, 1, 1);
     }
 #undef DAB_FCONV_LAUNCH
     DAB_LAUNCH_CHECK();
