@@ -188,6 +188,115 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
+// A few tiles only (256 and 512 input channels at batch 1 or 2): the kernel above would leave most SIMDs without a
+// wave, each of the few waves grinding through all 4 or 8 input words of 9 taps.  Here a block is one work item of 64
+// pixels x 8 output channels and its four waves split the depth: a channel's 18*CW weight dwords (9 taps x CW words,
+// contiguous) are 36 chunks of CW*2 bytes, four per tap, and wave w takes chunks [9w, 9w + 9) -- of the weights and
+// of every pixel's activations alike.  The block first copies the item's weights to LDS with coalesced loads (a
+// wave's share of a channel is too short and too strided for the scalar-load stream of the big kernel), the four
+// partial counts meet in LDS and the first wave applies the epilogue.  Eight channels are one byte of sign bits, so
+// the packed copy needs no coordination between blocks.
+template <int CW, int MODE>
+__global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p) {
+    constexpr int K32 = 18 * CW;       // weight dwords per channel
+    constexpr int CD = CW / 2;         // dwords per chunk (2 or 4)
+    constexpr int WD = 9 * CD;         // dwords per wave and channel
+    static_assert(CW == 4 || CW == 8, "256 or 512 input channels");
+    __shared__ __attribute__((aligned(16))) uint32_t wlds[8 * K32];
+    __shared__ uint32_t part[4][8][64];  // [wave][channel][pixel]
+    const int lane = threadIdx.x & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int tile = (int)p.div_groups.div(blockIdx.x);  // n_groups = cout / 8 here
+    const int cg = (int)blockIdx.x - tile * p.n_groups;
+
+    // the item's weights: 8 channels x K32 dwords, contiguous in memory
+    {
+        const uint64_t *wsrc = p.w + (size_t)cg * 8 * 9 * CW;
+        uint64_t *wdst = reinterpret_cast<uint64_t *>(wlds);
+        for (int i = threadIdx.x; i < 8 * 9 * CW; i += 256) wdst[i] = wsrc[i];
+    }
+
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
+    const int real_pix = tile * 64 + lane;
+    const int pix = real_pix < p.total ? real_pix : p.total - 1;
+    const uint32_t t = p.div_ow.div(pix);
+    const int ox = pix - t * p.OW;
+    const uint32_t n = p.div_oh.div(t);
+    const int oy = t - n * p.OH;
+    const int y0 = oy * p.stride - p.pad, x0 = ox * p.stride - p.pad;
+    const int base = ((n * p.H + y0) * p.W + x0) * (CW * 8);  // byte offset of tap (0,0); may be negative
+    uint32_t a[WD];
+#pragma unroll
+    for (int j = 0; j < 9; ++j) {
+        const int chunk = wib * 9 + j;  // wave-uniform
+        const int tap = chunk >> 2, kh = tap / 3, kw = tap - kh * 3;
+        const bool ok = (unsigned)(y0 + kh) < (unsigned)p.H && (unsigned)(x0 + kw) < (unsigned)p.W;
+        // beyond the descriptor's range a load returns zero: the reference's padding word
+        const int off = ok ? base + (kh * p.W + kw) * (CW * 8) + (chunk & 3) * (CD * 4) : (int)0x80000000;
+        if constexpr (CD == 2) {
+            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+            a[j * 2] = v.x, a[j * 2 + 1] = v.y;
+        } else {
+            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+            a[j * 4] = v.x, a[j * 4 + 1] = v.y, a[j * 4 + 2] = v.z, a[j * 4 + 3] = v.w;
+        }
+    }
+    __syncthreads();  // weights in LDS
+    const uint32_t *wq = wlds + wib * WD;  // this wave's quarter of channel 0; every lane reads the same words
+#pragma unroll
+    for (int ch = 0; ch < 8; ++ch) {
+        uint32_t c = 0;
+#pragma unroll
+        for (int d = 0; d < WD; ++d) c += __builtin_popcount(wq[ch * K32 + d] ^ a[d]);
+        part[wib][ch][lane] = c;
+    }
+    __syncthreads();
+    if (wib != 0 || real_pix >= p.total) return;
+
+    float v[8];
+#pragma unroll
+    for (int ch = 0; ch < 8; ++ch)
+        v[ch] = (float)(part[0][ch][lane] + part[1][ch][lane] + part[2][ch][lane] + part[3][ch][lane]);
+    const size_t off = (size_t)real_pix * p.cout + cg * 8;
+    if constexpr (MODE != kModeCounts) {
+#pragma clang fp contract(off)
+        // a*cnt + b (+ shortcut), each operation rounded on its own like the separate layers
+#pragma unroll
+        for (int ch = 0; ch < 8; ++ch) {
+            const float prod = p.epi_a[cg * 8 + ch] * v[ch];
+            v[ch] = prod + p.epi_b[cg * 8 + ch];
+        }
+        if (p.epi_shortcut != nullptr) {
+            const float4 s0 = *reinterpret_cast<const float4 *>(p.epi_shortcut + off);
+            const float4 s1 = *reinterpret_cast<const float4 *>(p.epi_shortcut + off + 4);
+            v[0] = v[0] + s0.x, v[1] = v[1] + s0.y, v[2] = v[2] + s0.z, v[3] = v[3] + s0.w;
+            v[4] = v[4] + s1.x, v[5] = v[5] + s1.y, v[6] = v[6] + s1.z, v[7] = v[7] + s1.w;
+        }
+    }
+    *reinterpret_cast<float4 *>(p.out + off) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(p.out + off + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    if constexpr (MODE == kModeAffineAddSign) {
+        uint32_t bits = 0;
+#pragma unroll
+        for (int ch = 0; ch < 8; ++ch) bits |= (v[ch] > 0.f ? 1u : 0u) << ch;
+        p.epi_bits[(size_t)real_pix * (p.cout >> 3) + cg] = (unsigned char)bits;
+    }
+}
+
+// So few work items (64 pixels x 8 channels) that splitting each over four waves still leaves SIMDs free.
+static bool splits_depth(long long tiles, int cin, int cout) {
+    return cin >= 256 && tiles * (cout / 8) * 4 <= simd_count();
+}
+
+template <int CW, int MODE>
+static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
+    a.n_groups = a.cout / 8;
+    a.div_groups = FastDiv((uint32_t)a.n_groups);
+    hipLaunchKernelGGL((bconv3x3_ksplit_kernel<CW, MODE>), dim3((unsigned)(tiles * a.n_groups)), dim3(256), 0, stream, a);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
 template <int CW, int MODE, bool NARROW>
 static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW>::value;
@@ -207,6 +316,9 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
+    if constexpr (CW >= 4) {
+        if (splits_depth(tiles, CW * 64, a.cout)) return launch_ksplit<CW, MODE>(a, tiles, stream);
+    }
     if constexpr (CW <= 2) {
         // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (a.cout / UnitChannels<CW>::value);
@@ -295,4 +407,9 @@ extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int
                                             float *out, uint64_t *out_packed, dab_stream_t stream) {
     return bconv3x3_impl("dab_bconv3x3_affine_add_sign", x, n, h, w, cin, wgt, cout, stride, pad, a, b, shortcut,
                          dab::kModeAffineAddSign, out, out_packed, stream);
+}
+
+extern "C" int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout) {
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 256 || cin == 512)) return 0;
+    return dab::splits_depth((n_out_pixels + 63) / 64, cin, cout) ? 1 : 0;
 }

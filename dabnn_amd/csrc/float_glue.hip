@@ -298,6 +298,50 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     }
 }
 
+// The classifier at small batch: a 1x1 convolution over a handful of pixels is a matrix-vector product, and the
+// 32 x 32 tiles above would leave all but 32 blocks idle.  One wave per output channel: lanes stride over the depth
+// with 16-byte loads (c % 4 == 0), the partial sums are added across the wave, lane 0 applies the epilogue.
+__global__ __launch_bounds__(256) void fconv_gemv_kernel(const FconvArgs p) {
+    constexpr int MR = 4;  // pixels that share one pass over a weight row
+    const int lane = threadIdx.x & 63;
+    const int co = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (co >= p.cout) return;
+    const float4 *w4 = reinterpret_cast<const float4 *>(p.w + (size_t)co * p.K);
+    const int k4n = p.K >> 2;
+    for (int m0 = 0; m0 < p.M; m0 += MR) {
+        float acc[MR] = {0.f, 0.f, 0.f, 0.f};
+        for (int k4 = lane; k4 < k4n; k4 += 64) {
+            const float4 wv = w4[k4];
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                const int m = m0 + r < p.M ? m0 + r : p.M - 1;  // a valid row; its sum is not stored
+                const float4 xv = reinterpret_cast<const float4 *>(p.x + (size_t)m * p.K)[k4];
+                acc[r] += wv.x * xv.x + wv.y * xv.y + wv.z * xv.z + wv.w * xv.w;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) acc[r] += __shfl_xor(acc[r], d, 64);
+        }
+        if (lane == 0) {
+#pragma clang fp contract(off)
+#pragma unroll
+            for (int r = 0; r < MR; ++r) {
+                if (m0 + r >= p.M) break;
+                float v = acc[r];
+                if (p.bias) v = v + p.bias[co];
+                if (p.aff_a) {
+                    const float prod = p.aff_a[co] * v;
+                    v = prod + p.aff_b[co];
+                }
+                if (p.relu) v = v > 0.f ? v : 0.f;
+                p.out[(size_t)(m0 + r) * p.cout + co] = v;
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- elementwise
 // Affine.cpp:10-23.  Multiply and add are kept as two roundings, as the
 // reference's x86 build does, so results match it bit for bit.
@@ -524,7 +568,14 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
     const int taps = kh * kw;
     const bool vec4 = c % 4 == 0 && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt)) % 16 == 0;
     const bool vec3 = c == 3 && bn == 64 && (taps + 7) / 8 * 24 * 10 <= (a.K + 15) / 16 * 16 * 11;
-    if (big_tiles < simd_count() / 4) {
+    if (M <= 8 && kh == 1 && kw == 1 && pad_h == 0 && pad_w == 0 && stride_h == 1 && stride_w == 1 && vec4 && cout >= 64) {
+        // a matrix-vector product (the classifier at small batch): one wave per output channel
+        hipLaunchKernelGGL(fconv_gemv_kernel, dim3((unsigned)((cout + 3) / 4)), dim3(256), 0, s, a);
+    } else if (big_tiles < simd_count() / 4 && vec3 && (M + 63) / 64 >= simd_count() / 8) {
+        // a three-channel image too small for 128-pixel tiles (the stem at batch 1): 64-pixel tiles keep the
+        // one-load-per-tap loader and still give most CUs a block
+        DAB_FCONV_LAUNCH(64, 64, 24, 1, 3);
+    } else if (big_tiles < simd_count() / 4) {
         // fewer big tiles than CUs: 32 x 32 tiles, each slice's depth split over the block's waves
         if (vec4)
             DAB_FCONV_LAUNCH(32, 32, 64, 4, 4);
@@ -653,19 +704,28 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
         const unsigned vb = (v.total + 255u) / 256u;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         float4 *o4 = reinterpret_cast<float4 *>(out);
-        const int taps = kh * kw;  // loads kept in flight: the whole window up to 3x3, 16 at a time beyond
+        // loads kept in flight: the whole window up to 3x3, 16 at a time beyond, 32 when the launch is too small to
+        // fill the chip and the chain of waits is all there is to it
+        const int taps = kh * kw;
+        const int batch_taps = taps <= 4 ? 4 : taps <= 9 ? 9 : (taps <= 16 || v.total > 65536u) ? 16 : 32;
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, out_packed, v);
         };
-        if (want_sign)
-            taps <= 4 ? launch(pool_vec4_kernel<true, true, 4>) : taps <= 9 ? launch(pool_vec4_kernel<true, true, 9>)
-                                                                            : launch(pool_vec4_kernel<true, true, 16>);
-        else if (is_max)
-            taps <= 4 ? launch(pool_vec4_kernel<true, false, 4>) : taps <= 9 ? launch(pool_vec4_kernel<true, false, 9>)
-                                                                             : launch(pool_vec4_kernel<true, false, 16>);
-        else
-            taps <= 4 ? launch(pool_vec4_kernel<false, false, 4>) : taps <= 9 ? launch(pool_vec4_kernel<false, false, 9>)
-                                                                              : launch(pool_vec4_kernel<false, false, 16>);
+#define DAB_POOL_LAUNCH(MAX, SIGN)                                               \
+    switch (batch_taps) {                                                        \
+        case 4: launch(pool_vec4_kernel<MAX, SIGN, 4>); break;                   \
+        case 9: launch(pool_vec4_kernel<MAX, SIGN, 9>); break;                   \
+        case 16: launch(pool_vec4_kernel<MAX, SIGN, 16>); break;                 \
+        default: launch(pool_vec4_kernel<MAX, SIGN, 32>); break;                 \
+    }
+        if (want_sign) {
+            DAB_POOL_LAUNCH(true, true)
+        } else if (is_max) {
+            DAB_POOL_LAUNCH(true, false)
+        } else {
+            DAB_POOL_LAUNCH(false, false)
+        }
+#undef DAB_POOL_LAUNCH
         DAB_LAUNCH_CHECK();
         return DAB_OK;
     }

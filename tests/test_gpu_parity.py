@@ -311,6 +311,9 @@ RTOL = 1e-4
     # padding, stride 1 and 2, dilation (the 7x7 cases take the one-load-per-tap loader)
     (5, 180, 3, 40, 7, 3, 2, 1, True), (5, 181, 3, 64, 7, 0, 2, 1, False), (2, 150, 3, 33, 7, 3, 1, 1, False),
     (4, 200, 3, 64, 7, 6, 2, 2, True), (4, 190, 3, 24, 3, 1, 2, 1, True),
+    # a handful of pixels through a 1x1 convolution: the matrix-vector kernel (ragged channel count, 1 to 8 pixels)
+    (1, 1, 512, 1000, 1, 0, 1, 1, True), (8, 1, 64, 70, 1, 0, 1, 1, False), (2, 2, 256, 65, 1, 0, 1, 1, True),
+    (5, 1, 1024, 64, 1, 0, 1, 1, False),
 ])
 def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
     r = rng(40)

@@ -159,10 +159,10 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     logits = n.get_blob("logits").reshape(2, -1)
     assert logits.shape == (2, 1000)
     descs = n.layers()
-    # the max pool and every block up to the first one with 512 input channels hand their successor the packed input;
-    # the three Adds of the down-sampling
-    # blocks are fused too, behind their shortcut branch
-    assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from its producer" in d for d in descs) == 14
+    # the max pool and every block hand their successor the packed input (at this batch the blocks with 512 input
+    # channels run the small-problem kernel, whose work items are whole bytes of sign bits); the three Adds of the
+    # down-sampling blocks are fused too, behind their shortcut branch
+    assert sum("+ Sign" in d for d in descs) == 15 and sum("packed input from its producer" in d for d in descs) == 16
     assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
     for i in range(2):
         assert check_every_segment(n, layers, inits, i) >= 20
@@ -174,6 +174,11 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     report = n.time_report()
     assert "Bin Conv" in report and "Float Conv" in report and "total" in report
     n.close()
+    # at a larger batch the two producers with 512 input channels leave the packing to their successors
+    big = net.Net(batch=16).read(str(path))
+    descs = big.layers()
+    assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from its producer" in d for d in descs) == 14
+    big.close()
 
 
 def test_error_paths(mods, tmp_path):
