@@ -209,6 +209,23 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
     const int tile = (int)p.div_groups.div(blockIdx.x);  // n_groups = cout / 8 here
     const int cg = (int)blockIdx.x - tile * p.n_groups;
 
+    // The first wave will need the epilogue's operands at the very end; asked for now, they arrive while the counts
+    // are made instead of adding a round trip to memory behind them.
+    const int real_pix = tile * 64 + lane;
+    const size_t out_off = (size_t)(real_pix < p.total ? real_pix : p.total - 1) * p.cout + cg * 8;
+    float ea[8], eb[8];
+    float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
+    if constexpr (MODE != kModeCounts) {
+        if (wib == 0) {
+#pragma unroll
+            for (int ch = 0; ch < 8; ++ch) ea[ch] = p.epi_a[cg * 8 + ch], eb[ch] = p.epi_b[cg * 8 + ch];
+            if (p.epi_shortcut != nullptr) {
+                s0 = *reinterpret_cast<const float4 *>(p.epi_shortcut + out_off);
+                s1 = *reinterpret_cast<const float4 *>(p.epi_shortcut + out_off + 4);
+            }
+        }
+    }
+
     // the item's weights: 8 channels x K32 dwords, contiguous in memory
     {
         const uint64_t *wsrc = p.w + (size_t)cg * 8 * 9 * CW;
@@ -217,7 +234,6 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
     }
 
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
-    const int real_pix = tile * 64 + lane;
     const int pix = real_pix < p.total ? real_pix : p.total - 1;
     const uint32_t t = p.div_ow.div(pix);
     const int ox = pix - t * p.OW;
@@ -257,24 +273,21 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
 #pragma unroll
     for (int ch = 0; ch < 8; ++ch)
         v[ch] = (float)(part[0][ch][lane] + part[1][ch][lane] + part[2][ch][lane] + part[3][ch][lane]);
-    const size_t off = (size_t)real_pix * p.cout + cg * 8;
     if constexpr (MODE != kModeCounts) {
 #pragma clang fp contract(off)
         // a*cnt + b (+ shortcut), each operation rounded on its own like the separate layers
 #pragma unroll
         for (int ch = 0; ch < 8; ++ch) {
-            const float prod = p.epi_a[cg * 8 + ch] * v[ch];
-            v[ch] = prod + p.epi_b[cg * 8 + ch];
+            const float prod = ea[ch] * v[ch];
+            v[ch] = prod + eb[ch];
         }
         if (p.epi_shortcut != nullptr) {
-            const float4 s0 = *reinterpret_cast<const float4 *>(p.epi_shortcut + off);
-            const float4 s1 = *reinterpret_cast<const float4 *>(p.epi_shortcut + off + 4);
             v[0] = v[0] + s0.x, v[1] = v[1] + s0.y, v[2] = v[2] + s0.z, v[3] = v[3] + s0.w;
             v[4] = v[4] + s1.x, v[5] = v[5] + s1.y, v[6] = v[6] + s1.z, v[7] = v[7] + s1.w;
         }
     }
-    *reinterpret_cast<float4 *>(p.out + off) = make_float4(v[0], v[1], v[2], v[3]);
-    *reinterpret_cast<float4 *>(p.out + off + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    *reinterpret_cast<float4 *>(p.out + out_off) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(p.out + out_off + 4) = make_float4(v[4], v[5], v[6], v[7]);
     if constexpr (MODE == kModeAffineAddSign) {
         uint32_t bits = 0;
 #pragma unroll
