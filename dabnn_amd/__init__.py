@@ -12,6 +12,7 @@ from .ops import (  # noqa: F401
     add_inplace,
     affine_inplace,
     ave_pool,
+    ave_pool2_fconv1x1,
     bconv_3x3,
     bconv_3x3_affine_add,
     bconv_3x3_affine_add_sign,

@@ -57,6 +57,7 @@ SIGNATURES = {
     "dab_binconv_forward": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 8 + [_vp, _vp, _sz, ctypes.POINTER(_i), _vp]),
     "dab_fconv": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 9 + [_vp, _vp]),
     "dab_fconv_affine_relu": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp] + [_i] * 10 + [_vp, _vp]),
+    "dab_ave_pool2_fconv1x1": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
     "dab_affine_inplace": (_i, [_vp, _i64, _i, _vp, _vp, _vp]),
     "dab_add_inplace": (_i, [_vp, _vp, _i64, _vp]),
     "dab_relu_inplace": (_i, [_vp, _i64, _vp]),

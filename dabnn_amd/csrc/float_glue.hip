@@ -32,7 +32,10 @@ namespace dab {
 // the three channels of one tap with one 12-byte load, so a slice (8 taps = 24
 // depths) takes a third of the load instructions and of the address and bounds
 // arithmetic per depth.  CV = 4 does the same with 16-byte loads of four
-// consecutive channels when the channel count is a multiple of 4.
+// consecutive channels when the channel count is a multiple of 4.  POOL (1x1
+// convolutions with CV = 4) averages 2x2 windows of the input on the way in --
+// an AvePool 2x2 stride 2 followed by the convolution, the shortcut branch of a
+// down-sampling block, in one launch; the pooled tensor is still written.
 struct FconvArgs {
     const float *x;
     const float *w;
@@ -40,6 +43,7 @@ struct FconvArgs {
     const float *aff_a;
     const float *aff_b;
     float *out;
+    float *pooled;  // POOL kernels: the 2x2-averaged input, written as a side product
     int n, h, wd, c;
     int kw, dil_h, dil_w;
     int pad_h, pad_w, stride_h, stride_w;
@@ -59,7 +63,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr uint32_t kOob = 0x80000000u;     // descriptors here are shorter than 2^30 bytes
 constexpr uint32_t kOobRow = 0x40000000u;  // kOobRow + kOob and kOobRow + (anything < 2^30) stay out of range
 
-template <int BM, int BN, int SK, int KSPLIT, bool PADDED, int CV = 1>
+template <int BM, int BN, int SK, int KSPLIT, bool PADDED, int CV = 1, bool POOL = false>
 __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     constexpr int WAVES_MN = 4 / KSPLIT;
     constexpr int WAVES_N = (WAVES_MN >= 2 && BN >= 64) ? 2 : 1, WAVES_M = WAVES_MN / WAVES_N;
@@ -73,6 +77,8 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert(WK % 8 == 0 && 256 % LK == 0 && APT >= 1 && BPT >= 1, "slice");
     static_assert(CV == 1 || CV == 4 || (CV == 3 && KSPLIT == 1), "channel-vector loader");
+    static_assert(!POOL || (CV == 4 && !PADDED), "the pooling loader takes whole 2x2 windows of four channels");
+    constexpr int NW = POOL ? 4 : 1;  // loads per tile element: the window of the pooled input
     constexpr bool B_PARTIAL = BN < RP;  // fewer weight rows than loader rows: the upper loader rows fetch nothing
     __shared__ __attribute__((aligned(16))) float As[2][BM][RS];
     __shared__ __attribute__((aligned(16))) float Bs[2][BN][RS];
@@ -137,7 +143,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     for (int j = 0; j < BPT; ++j) b_row[j] = (uint32_t)(l_r + RP * j) * p.K * 4u;
 
     typedef float f32xcv __attribute__((ext_vector_type(CV)));
-    f32xcv a_reg[APT], b_reg[BPT];
+    f32xcv a_reg[APT][NW], b_reg[BPT];
     auto load_cv = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off) -> f32xcv {
         // the result is bit-cast as a whole: casting single elements of a vector buffer load makes the compiler
         // replace it by one 4-byte load
@@ -169,17 +175,41 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
                 const int y = a_y0[i] + dy, xx = a_x0[i] + dx;
                 off = ((unsigned)y < (unsigned)p.h && (unsigned)xx < (unsigned)p.wd) ? off : kOob;
             }
-            a_reg[i] = load_cv(x_rsrc, off);
+            a_reg[i][0] = load_cv(x_rsrc, off);
+            if constexpr (POOL) {
+                // the window's other three pixels: right, below, below right (out-of-range elements carry kOob and
+                // stay out of range with these small additions)
+                const uint32_t right = (uint32_t)p.c * 4u, below = (uint32_t)p.wd * right;
+                a_reg[i][1] = load_cv(x_rsrc, off + right);
+                a_reg[i][2] = load_cv(x_rsrc, off + below);
+                a_reg[i][3] = load_cv(x_rsrc, off + below + right);
+            }
         }
         const uint32_t k4 = k_ok ? (uint32_t)k * 4u : kOob;
 #pragma unroll
         for (int j = 0; j < BPT; ++j) b_reg[j] = load_cv(w_rsrc, (!B_PARTIAL || l_r < BN) ? b_row[j] + k4 : kOob);
     };
-    auto commit = [&](int buf) {
+    auto commit = [&](int buf, int k0) {
 #pragma unroll
-        for (int i = 0; i < APT; ++i)
+        for (int i = 0; i < APT; ++i) {
+            f32xcv v = a_reg[i][0];
+            if constexpr (POOL) {
+                // ave_pool_fallback (dabnn/layers/AvePool.cpp:84-123) for a 2x2 window without padding: the taps are
+                // added to zero in row-major order and divided by 4 (a multiplication by 0.25 rounds the same way)
+#pragma clang fp contract(off)
+                f32xcv sum = {0.f, 0.f, 0.f, 0.f};
+                sum = sum + a_reg[i][0];
+                sum = sum + a_reg[i][1];
+                sum = sum + a_reg[i][2];
+                sum = sum + a_reg[i][3];
+                v = sum * 0.25f;
+                const int pix = m0 + l_r + RP * i, k = k0 + CV * l_k;
+                if (blockIdx.y == 0 && pix < p.M && k < p.K)
+                    *reinterpret_cast<f32xcv *>(p.pooled + (size_t)pix * p.K + k) = v;
+            }
 #pragma unroll
-            for (int c = 0; c < CV; ++c) As[buf][l_r + RP * i][l_k * CV + c] = a_reg[i][c];
+            for (int c = 0; c < CV; ++c) As[buf][l_r + RP * i][l_k * CV + c] = v[c];
+        }
         if (!B_PARTIAL || l_r < BN) {
 #pragma unroll
             for (int j = 0; j < BPT; ++j)
@@ -199,7 +229,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     // operand lane l of the instruction: row / column l % 32, depth slot l / 32
     const int f_k = lane >> 5, f_i = lane & 31;
     fetch(0);
-    commit(0);
+    commit(0, 0);
     __syncthreads();
     int buf = 0;
     for (int k0 = 0; k0 < p.K; k0 += SK, buf ^= 1) {
@@ -224,7 +254,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
                 }
         }
         // the other buffer was last read before the barrier that ended the previous slice
-        if (more) commit(buf ^ 1);
+        if (more) commit(buf ^ 1, k0 + SK);
         __syncthreads();
     }
 
@@ -530,6 +560,7 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
     DAB_REQUIRE((aff_a == nullptr) == (aff_b == nullptr), "%s: affine needs both coefficient vectors", fn);
     FconvArgs a;
     a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.relu = relu, a.out = out;
+    a.pooled = nullptr;
     a.n = n, a.h = h, a.wd = w, a.c = c;
     a.pad_h = pad_h, a.pad_w = pad_w, a.stride_h = stride_h, a.stride_w = stride_w;
     a.oh = out_dim(h, pad_h, kh, dil_h, stride_h), a.ow = out_dim(w, pad_w, kw, dil_w, stride_w);
@@ -600,6 +631,53 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
             DAB_FCONV_LAUNCH(128, 128, 16, 1, 1);
     }
 #undef DAB_FCONV_LAUNCH
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                      const float *aff_a, const float *aff_b, int relu, int cout, float *pooled, float *out,
+                                      dab_stream_t stream) {
+    using namespace dab;
+    const char *fn = "dab_ave_pool2_fconv1x1";
+    DAB_REQUIRE(x && wgt && pooled && out, "%s: null pointer", fn);
+    DAB_REQUIRE(n > 0 && h >= 2 && w >= 2 && c > 0 && cout > 0, "%s: bad dimension (the input must hold a 2x2 window)", fn);
+    DAB_REQUIRE((aff_a == nullptr) == (aff_b == nullptr), "%s: affine needs both coefficient vectors", fn);
+    if (c % 4 != 0 ||
+        (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt) | reinterpret_cast<uintptr_t>(pooled)) % 16 != 0)
+        return fail(DAB_EUNSUPPORTED, "%s: needs c %% 4 == 0 and 16-byte aligned buffers", fn);
+    FconvArgs a;
+    a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.relu = relu, a.out = out, a.pooled = pooled;
+    a.n = n, a.h = h, a.wd = w, a.c = c;
+    a.pad_h = 0, a.pad_w = 0, a.stride_h = 2, a.stride_w = 2;  // a pooled pixel's window starts at twice its coordinates
+    a.oh = out_dim(h, 0, 2, 1, 2), a.ow = out_dim(w, 0, 2, 1, 2);
+    a.cout = cout;
+    a.K = c;
+    const long long M = (long long)n * a.oh * a.ow;
+    if (M >= (1ll << 31) - 128 || (long long)n * h * w * c >= (1ll << 31))
+        return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
+    a.M = (int)M;
+    a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
+    a.kw = 1, a.dil_h = 1, a.dil_w = 1;
+    a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv(1u);
+    const long long span_imgs = 128 / ((long long)a.oh * a.ow) + 2;
+    if (span_imgs * h * w * c * 4 >= (1ll << 30) || 128ll * a.K * 4 >= (1ll << 30) || 128ll * cout * 4 >= (1ll << 30))
+        return fail(DAB_EUNSUPPORTED, "%s: image, filter or channel count too large for 32-bit tile offsets", fn);
+    hipStream_t s = as_stream(stream);
+    const int bn = cout <= 32 ? 32 : cout <= 64 ? 64 : 128;
+    const long long big_tiles = ((M + 127) / 128) * ((cout + bn - 1) / bn);
+#define DAB_POOLED_LAUNCH(BM, BN, SK, KSPLIT)                                                                     \
+    hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false, 4, true>),                                        \
+                       dim3((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN)), dim3(256), 0, s, a)
+    if (big_tiles < simd_count() / 4)
+        DAB_POOLED_LAUNCH(32, 32, 64, 4);
+    else if (bn == 32)
+        DAB_POOLED_LAUNCH(128, 32, 16, 1);
+    else if (bn == 64)
+        DAB_POOLED_LAUNCH(128, 64, 16, 1);
+    else
+        DAB_POOLED_LAUNCH(128, 128, 16, 1);
+#undef DAB_POOLED_LAUNCH
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }

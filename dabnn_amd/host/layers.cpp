@@ -161,6 +161,16 @@ FloatConv::FloatConv(NetCP net, css name, css input, css weight, css output, int
       dilation(dilation_) {}
 
 void FloatConv::forward_impl() const {
+    if (fused_pool_input) {
+        dab_check(dab_ave_pool2_fconv1x1(
+            static_cast<const float *>(fused_pool_input->data), fused_pool_input->n, fused_pool_input->h, fused_pool_input->w,
+            fused_pool_input->c, static_cast<const float *>(weight_mat->data),
+            bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
+            fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
+            fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, output_mat->c,
+            static_cast<float *>(input_mat->data), static_cast<float *>(output_mat->data), stream()));
+        return;
+    }
     dab_check(dab_fconv_affine_relu(
         static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
         static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
@@ -176,6 +186,7 @@ std::string FloatConv::to_str() const {
        << "x" << weight_mat->h << "x" << weight_mat->w;
     if (fused_a) ss << " + Affine";
     if (fused_relu) ss << " + Relu";
+    if (fused_pool_input) ss << ", AvePool 2x2 of " << fused_pool_input->h << "x" << fused_pool_input->w << " inside";
     return ss.str();
 }
 

@@ -47,6 +47,9 @@ class FloatConv : public Layer {
     // Affine (and Relu) layers that follow on the output blob, applied in the convolution's epilogue when set
     MatP fused_a, fused_b;
     bool fused_relu = false;
+    // Set by Net::prepare for a 1x1 convolution that reads the output of an AvePool 2x2 stride 2: the pool's input.
+    // The layer then pools it itself, writes the pooled blob (input_mat) as a side product and convolves it.
+    MatP fused_pool_input;
     const int pad_h, pad_w, stride_h, stride_w, dilation;
     FloatConv(NetCP net, css name, css input, css weight, css bias, css output, int pad_h, int pad_w, int stride_h,
               int stride_w, int dilation);

@@ -310,8 +310,9 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
         reads = {bc->input_mat.get()};
         writes = {bc->output_mat.get(), bc->binarized_mat.get(), bc->col_mat.get()};
     } else if (auto fc = std::dynamic_pointer_cast<FloatConv>(l)) {
-        reads = {fc->input_mat.get()};
+        reads = {fc->fused_pool_input ? fc->fused_pool_input.get() : fc->input_mat.get()};
         writes = {fc->output_mat.get()};
+        if (fc->fused_pool_input) writes.push_back(fc->input_mat.get());  // the pooled blob, a side product
     } else if (auto af = std::dynamic_pointer_cast<Affine>(l)) {
         reads = writes = {af->data_mat.get()};
     } else if (auto ad = std::dynamic_pointer_cast<Add>(l)) {
@@ -348,6 +349,8 @@ static bool contains(const std::vector<const Mat *> &v, const Mat *m) {
 //     one pass of the float convolution.
 //  3. When the blob such a fused BinConv completes is the input of a later direct BinConv, the pass also writes that
 //     layer's packed input and the later layer skips its pack_mat.
+//  4. AvePool 2x2 stride 2 -> 1x1 FloatConv (the shortcut branch of a down-sampling block) becomes one launch that
+//     still writes the pooled blob.
 void Net::fuse_binconv_epilogues() {
     std::vector<const Mat *> rd, wr;
     for (size_t i = 0; i + 2 < layers.size(); ++i) {
@@ -445,6 +448,34 @@ void Net::fuse_binconv_epilogues() {
             layer_io(layers[j], rd, wr);
             if (contains(wr, producer->output_mat.get())) break;  // the blob changes again before anyone packs it
         }
+    }
+
+    for (size_t i = 0; i + 1 < layers.size(); ++i) {
+        auto pool = std::dynamic_pointer_cast<AvePool>(layers[i]);
+        if (!pool || pool->kernel_h != 2 || pool->kernel_w != 2 || pool->stride_h != 2 || pool->stride_w != 2 ||
+            pool->pad_h != 0 || pool->pad_w != 0 || pool->input_mat->c % 4 != 0 || pool->input_mat->h < 2 ||
+            pool->input_mat->w < 2)
+            continue;
+        // the one reader of the pooled blob must be a 1x1 FloatConv, with nothing in between that rewrites the pool's input
+        size_t j = i + 1;
+        bool ok = true;
+        for (; j < layers.size(); ++j) {
+            layer_io(layers[j], rd, wr);
+            if (contains(rd, pool->output_mat.get())) break;
+            if (contains(wr, pool->input_mat.get()) || contains(wr, pool->output_mat.get())) ok = false;
+        }
+        auto fc = j < layers.size() ? std::dynamic_pointer_cast<FloatConv>(layers[j]) : nullptr;
+        if (!ok || !fc || fc->input_mat != pool->output_mat || fc->weight_mat->h != 1 || fc->weight_mat->w != 1 ||
+            fc->pad_h != 0 || fc->pad_w != 0 || fc->stride_h != 1 || fc->stride_w != 1 || fc->dilation != 1)
+            continue;
+        for (size_t k = j + 1; k < layers.size() && ok; ++k) {
+            layer_io(layers[k], rd, wr);
+            if (contains(rd, pool->output_mat.get())) ok = false;  // someone else wants the pooled blob at its own time
+        }
+        if (!ok) continue;
+        fc->fused_pool_input = pool->input_mat;
+        layers.erase(layers.begin() + i);
+        --i;
     }
 }
 

@@ -239,6 +239,29 @@ def fconv_affine_relu(x, weight, bias, a, b, relu, kh, kw, pad_h, pad_w, stride_
     return out
 
 
+def ave_pool2_fconv1x1(x, weight, bias, a, b, relu):
+    """AvePool 2x2 stride 2 + 1x1 FpConv2D (+ Affine + Relu) in one launch; returns (pooled, out)."""
+    _need(x, torch.float32, "x")
+    _need(weight, torch.float32, "weight")
+    n, h, w, c = x.shape
+    cout = weight.shape[0]
+    if weight.numel() != cout * c:
+        raise capi.DabError(capi.DAB_EINVAL, "ave_pool2_fconv1x1: weight must be [cout, 1, 1, c]")
+    def opt(t, name):
+        if t is None:
+            return None
+        _need(t, torch.float32, name)
+        if t.numel() != cout:
+            raise capi.DabError(capi.DAB_EINVAL, "ave_pool2_fconv1x1: %s does not match the channel count" % name)
+        return _ptr(t)
+    oh, ow = out_dim(h, 0, 2, 2), out_dim(w, 0, 2, 2)
+    pooled = _empty((n, max(oh, 0), max(ow, 0), c), torch.float32, x.device)
+    out = _empty((n, max(oh, 0), max(ow, 0), cout), torch.float32, x.device)
+    check(lib.dab_ave_pool2_fconv1x1(_ptr(x), n, h, w, c, _ptr(weight), opt(bias, "bias"), opt(a, "a"), opt(b, "b"),
+                                     int(bool(relu)), cout, _ptr(pooled), _ptr(out), _stream()))
+    return pooled, out
+
+
 def affine_inplace(x, a, b):
     """affine_inplace (dabnn/layers/Affine.cpp:10-23)."""
     _need(x, torch.float32, "x")

@@ -182,6 +182,17 @@ DAB_API int dab_fconv_affine_relu(const float *x, int n, int h, int w, int c, co
                                   int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *out,
                                   dab_stream_t stream);
 
+/*
+ * AvePool 2x2, stride 2, no padding (ave_pool_fallback, dabnn/layers/AvePool.cpp:84-123) followed by a 1x1 FpConv2D
+ * (dabnn/fconv.h:14-76) and the optional Affine and Relu of dab_fconv_affine_relu, in one launch: the shortcut branch
+ * of a down-sampling block.  pooled [n][(h-2)/2+1][(w-2)/2+1][c] receives the pooled tensor exactly as dab_ave_pool
+ * writes it, out the convolution of it exactly as dab_fconv_affine_relu computes it from that tensor.
+ * wgt is [cout][1][1][c].  c must be a multiple of 4 and x, wgt, pooled 16-byte aligned (DAB_EUNSUPPORTED otherwise).
+ */
+DAB_API int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                   const float *a, const float *b, int relu, int cout, float *pooled, float *out,
+                                   dab_stream_t stream);
+
 /* affine_inplace (dabnn/layers/Affine.cpp:10-23): x[..., ch] = a[ch]*x[..., ch] + b[ch]. */
 DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, const float *b, dab_stream_t stream);
 

@@ -386,6 +386,29 @@ def test_affine_add_bit_exact(dab):
     np.testing.assert_array_equal(got2, want + y)
 
 
+@pytest.mark.parametrize("n,h,w,c,cout,affine", [(1, 56, 56, 64, 128, True), (2, 9, 7, 8, 5, False), (3, 28, 28, 128, 256, True),
+                                                 (1, 14, 14, 256, 512, True), (40, 56, 56, 64, 128, True), (1, 2, 2, 4, 8, False)])
+def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine):
+    """The shortcut branch of a down-sampling block in one launch: the pooled tensor is bit for bit what ave_pool
+    writes (and what the CPU restatement computes), the convolution bit for bit what fconv_affine_relu makes of it."""
+    r = rng(46)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    x[0, 0, 0, :4] = [0.0, -0.0, 1e-40, -1e-40]
+    wgt = (r.standard_normal((cout, 1, 1, c)) / np.sqrt(c)).astype(np.float32)
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    pooled, out = dab.ave_pool2_fconv1x1(dev_f(x), dev_f(wgt), None, dev_f(a) if affine else None,
+                                         dev_f(b) if affine else None, False)
+    want_pooled = dab.ave_pool(dev_f(x), 2, 2, 0, 0, 2, 2)
+    want_out = dab.fconv_affine_relu(want_pooled, dev_f(wgt), None, dev_f(a) if affine else None,
+                                     dev_f(b) if affine else None, False, 1, 1, 0, 0, 1, 1)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want_pooled.cpu().numpy())
+    np.testing.assert_array_equal(out.cpu().numpy(), want_out.cpu().numpy())
+    cpu_pooled = np.stack([orc.ave_pool(img, 2, 2, 0, 0, 2, 2) for img in x[:2]])
+    np.testing.assert_array_equal(pooled.cpu().numpy()[:2], cpu_pooled)
+    with pytest.raises(RuntimeError):
+        dab.ave_pool2_fconv1x1(dev_f(x[..., :3].copy()), dev_f(wgt[..., :3].copy()), None, None, None, False)
+
+
 @pytest.mark.parametrize("shape", [(2, 5, 7, 64), (1, 3, 3, 5), (3, 16, 16, 192), (1, 1, 1, 1)])
 def test_prelu_bit_exact(dab, shape):
     r = rng(44)

@@ -164,6 +164,8 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     # down-sampling blocks are fused too, behind their shortcut branch
     assert sum("+ Sign" in d for d in descs) == 15 and sum("packed input from its producer" in d for d in descs) == 16
     assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
+    # the three shortcut branches pool inside their 1x1 convolution; only the global pool is left as a layer
+    assert sum("AvePool 2x2 of" in d for d in descs) == 3 and sum(d.startswith("AvePool") for d in descs) == 1
     for i in range(2):
         assert check_every_segment(n, layers, inits, i) >= 20
         assert check_packed_inputs(n, layers, i) == 16
