@@ -188,7 +188,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
-// A few tiles only (256 and 512 input channels at batch 1 or 2): the kernel above would leave most SIMDs without a
+// A few tiles only (128 to 512 input channels at batch 1 or 2): the kernel above would leave most SIMDs without a
 // wave, each of the few waves grinding through all 4 or 8 input words of 9 taps.  Here a block is one work item of 64
 // pixels x 8 output channels and its four waves split the depth: a channel's 18*CW weight dwords (9 taps x CW words,
 // contiguous) are 36 chunks of CW*2 bytes, four per tap, and wave w takes chunks [9w, 9w + 9) -- of the weights and
@@ -199,9 +199,9 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
 template <int CW, int MODE>
 __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;       // weight dwords per channel
-    constexpr int CD = CW / 2;         // dwords per chunk (2 or 4)
+    constexpr int CD = CW / 2;         // dwords per chunk (1, 2 or 4)
     constexpr int WD = 9 * CD;         // dwords per wave and channel
-    static_assert(CW == 4 || CW == 8, "256 or 512 input channels");
+    static_assert(CW == 2 || CW == 4 || CW == 8, "128, 256 or 512 input channels");
     __shared__ __attribute__((aligned(16))) uint32_t wlds[8 * K32];
     __shared__ uint32_t part[4][8][64];  // [wave][channel][pixel]
     const int lane = threadIdx.x & 63;
@@ -249,7 +249,9 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
         const bool ok = (unsigned)(y0 + kh) < (unsigned)p.H && (unsigned)(x0 + kw) < (unsigned)p.W;
         // beyond the descriptor's range a load returns zero: the reference's padding word
         const int off = ok ? base + (kh * p.W + kw) * (CW * 8) + (chunk & 3) * (CD * 4) : (int)0x80000000;
-        if constexpr (CD == 2) {
+        if constexpr (CD == 1) {
+            a[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
+        } else if constexpr (CD == 2) {
             const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
             a[j * 2] = v.x, a[j * 2 + 1] = v.y;
         } else {
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
 
 // So few work items (64 pixels x 8 channels) that splitting each over four waves still leaves SIMDs free.
 static bool splits_depth(long long tiles, int cin, int cout) {
-    return cin >= 256 && tiles * (cout / 8) * 4 <= simd_count();
+    return cin >= 128 && tiles * (cout / 8) * 4 <= simd_count();
 }
 
 template <int CW, int MODE>
@@ -329,7 +331,7 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
-    if constexpr (CW >= 4) {
+    if constexpr (CW >= 2) {
         if (splits_depth(tiles, CW * 64, a.cout)) return launch_ksplit<CW, MODE>(a, tiles, stream);
     }
     if constexpr (CW <= 2) {
@@ -423,6 +425,6 @@ extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int
 }
 
 extern "C" int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout) {
-    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 256 || cin == 512)) return 0;
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 128 || cin == 256 || cin == 512)) return 0;
     return dab::splits_depth((n_out_pixels + 63) / 64, cin, cout) ? 1 : 0;
 }
