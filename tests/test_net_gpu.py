@@ -177,7 +177,7 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     assert "Bin Conv" in report and "Float Conv" in report and "total" in report
     n.close()
     # at a larger batch the two producers with 512 input channels leave the packing to their successors
-    big = net.Net(batch=16).read(str(path))
+    big = net.Net(batch=32).read(str(path))
     descs = big.layers()
     assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from its producer" in d for d in descs) == 14
     big.close()
