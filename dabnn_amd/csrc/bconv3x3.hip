@@ -188,7 +188,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
-// A few tiles only (128 to 512 input channels at batch 1 or 2): the kernel above would leave most SIMDs without a
+// A few tiles only (small batches): the kernel above would leave most SIMDs without a
 // wave, each of the few waves grinding through all 4 or 8 input words of 9 taps.  Here a block is one work item of 64
 // pixels x 8 output channels and its four waves split the depth: a channel's 18*CW weight dwords (9 taps x CW words,
 // contiguous) are 36 chunks of CW*2 bytes, four per tap, and wave w takes chunks [9w, 9w + 9) -- of the weights and
@@ -200,8 +200,8 @@ template <int CW, int MODE>
 __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;       // weight dwords per channel
     constexpr int CD = CW / 2;         // dwords per chunk (1, 2 or 4)
-    constexpr int WD = 9 * CD;         // dwords per wave and channel
-    static_assert(CW == 2 || CW == 4 || CW == 8, "128, 256 or 512 input channels");
+    // dwords per wave and channel; with 64 input channels the 18 dwords of a channel go 5, 5, 4, 4 to the waves
+    constexpr int WD = CW == 1 ? 5 : 9 * CD;
     __shared__ __attribute__((aligned(16))) uint32_t wlds[8 * K32];
     __shared__ uint32_t part[4][8][64];  // [wave][channel][pixel]
     const int lane = threadIdx.x & 63;
@@ -242,30 +242,45 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
     const int y0 = oy * p.stride - p.pad, x0 = ox * p.stride - p.pad;
     const int base = ((n * p.H + y0) * p.W + x0) * (CW * 8);  // byte offset of tap (0,0); may be negative
     uint32_t a[WD];
+    const int first = CW == 1 ? wib * 5 - (wib > 2 ? wib - 2 : 0) : wib * WD;  // this wave's first dword of a channel
+    const int count = CW == 1 ? (wib < 2 ? 5 : 4) : WD;                         // and how many it takes
+    if constexpr (CW == 1) {
 #pragma unroll
-    for (int j = 0; j < 9; ++j) {
-        const int chunk = wib * 9 + j;  // wave-uniform
-        const int tap = chunk >> 2, kh = tap / 3, kw = tap - kh * 3;
-        const bool ok = (unsigned)(y0 + kh) < (unsigned)p.H && (unsigned)(x0 + kw) < (unsigned)p.W;
-        // beyond the descriptor's range a load returns zero: the reference's padding word
-        const int off = ok ? base + (kh * p.W + kw) * (CW * 8) + (chunk & 3) * (CD * 4) : (int)0x80000000;
-        if constexpr (CD == 1) {
-            a[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
-        } else if constexpr (CD == 2) {
-            const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
-            a[j * 2] = v.x, a[j * 2 + 1] = v.y;
-        } else {
-            const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
-            a[j * 4] = v.x, a[j * 4 + 1] = v.y, a[j * 4 + 2] = v.z, a[j * 4 + 3] = v.w;
+        for (int j = 0; j < WD; ++j) {
+            const int d = first + j;  // wave-uniform; two dwords per tap
+            const int tap = d >> 1, kh = tap / 3, kw = tap - kh * 3;
+            const bool ok = j < count && (unsigned)(y0 + kh) < (unsigned)p.H && (unsigned)(x0 + kw) < (unsigned)p.W;
+            // beyond the descriptor's range a load returns zero: the reference's padding word
+            a[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, ok ? base + (kh * p.W + kw) * 8 + (d & 1) * 4 : (int)0x80000000, 0, 0);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 9; ++j) {
+            const int chunk = wib * 9 + j;  // wave-uniform
+            const int tap = chunk >> 2, kh = tap / 3, kw = tap - kh * 3;
+            const bool ok = (unsigned)(y0 + kh) < (unsigned)p.H && (unsigned)(x0 + kw) < (unsigned)p.W;
+            const int off = ok ? base + (kh * p.W + kw) * (CW * 8) + (chunk & 3) * (CD * 4) : (int)0x80000000;
+            if constexpr (CD == 1) {
+                a[j] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, 0, 0);
+            } else if constexpr (CD == 2) {
+                const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
+                a[j * 2] = v.x, a[j * 2 + 1] = v.y;
+            } else {
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
+                a[j * 4] = v.x, a[j * 4 + 1] = v.y, a[j * 4 + 2] = v.z, a[j * 4 + 3] = v.w;
+            }
         }
     }
     __syncthreads();  // weights in LDS
-    const uint32_t *wq = wlds + wib * WD;  // this wave's quarter of channel 0; every lane reads the same words
+    const uint32_t *wq = wlds + first;  // this wave's share of channel 0; every lane reads the same words
 #pragma unroll
     for (int ch = 0; ch < 8; ++ch) {
         uint32_t c = 0;
 #pragma unroll
-        for (int d = 0; d < WD; ++d) c += __builtin_popcount(wq[ch * K32 + d] ^ a[d]);
+        for (int d = 0; d < WD; ++d) {
+            const uint32_t wd = (CW > 1 || d < count) ? wq[ch * K32 + d] : 0u;  // a[d] is zero where the share ends
+            c += __builtin_popcount(wd ^ a[d]);
+        }
         part[wib][ch][lane] = c;
     }
     __syncthreads();
@@ -301,7 +316,7 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
 // So few work items (64 pixels x 8 channels) that splitting each over four waves gives a SIMD four waves at most
 // (measured on Bi-Real-18 at batch 1 to 16: faster than the unit kernel up to there).
 static bool splits_depth(long long tiles, int cin, int cout) {
-    return cin >= 128 && tiles * (cout / 8) <= simd_count();
+    return tiles * (cout / 8) <= simd_count();
 }
 
 template <int CW, int MODE>
@@ -332,9 +347,7 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
-    if constexpr (CW >= 2) {
-        if (splits_depth(tiles, CW * 64, a.cout)) return launch_ksplit<CW, MODE>(a, tiles, stream);
-    }
+    if (splits_depth(tiles, CW * 64, a.cout)) return launch_ksplit<CW, MODE>(a, tiles, stream);
     if constexpr (CW <= 2) {
         // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (a.cout / UnitChannels<CW>::value);
@@ -426,6 +439,6 @@ extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int
 }
 
 extern "C" int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout) {
-    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 128 || cin == 256 || cin == 512)) return 0;
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return 0;
     return dab::splits_depth((n_out_pixels + 63) / 64, cin, cout) ? 1 : 0;
 }

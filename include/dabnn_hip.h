@@ -139,7 +139,7 @@ DAB_API int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int w,
 /*
  * No counterpart in the reference: 1 when dab_bconv3x3* would run this problem (n_out_pixels = N*OH*OW) with its
  * small-problem kernel, whose work items are whole bytes of sign bits -- dab_bconv3x3_affine_add_sign then costs no
- * more than dab_bconv3x3_affine_add, also for 512 input channels (cin 128, 256 or 512; other values answer 0), where the large kernel makes the packed copy
+ * more than dab_bconv3x3_affine_add, also for 512 input channels (cin 64, 128, 256 or 512; other values answer 0), where the large kernel makes the packed copy
  * dearer than a separate dab_bitpack_nhwc.  0 otherwise.  Net::prepare uses it to decide which layers to link.
  */
 DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
