@@ -222,6 +222,21 @@ def main():
         layers, inits, inputs = models.bireal18(2024, stem=stem)
         model_cache[stem] = (layers, inits)
         buf = dab_format.write_model(layers, inits, inputs)
+        if not stem:
+            # batches in between, images/s only (graph replay, input on the device)
+            sweep = {}
+            for batch in (2, 4, 8, 16, 64):
+                net = dabnet.Net(batch=batch).read_buf(buf)
+                x = torch.randn((batch, 224, 224, 3), generator=g).cuda()
+                for _ in range(3):
+                    net.run(x)
+                t1 = time.perf_counter()
+                for _ in range(20):
+                    net.run(x)
+                sweep["b%d" % batch] = round(batch * 20 / (time.perf_counter() - t1), 1)
+                net.close()
+                del x
+            bireal["bireal18_images_per_s_by_batch"] = sweep
         for batch in (1, 256):
             net = dabnet.Net(batch=batch).read_buf(buf)
             x = torch.randn((batch, 224, 224, 3), generator=g).cuda()
