@@ -22,6 +22,8 @@ from .ops import (  # noqa: F401
     concat,
     fconv,
     fconv_affine_relu,
+    fconv_maxpool,
+    fconv_maxpool_pays,
     fused_binarize_im2col,
     max_pool,
     max_pool_sign,

@@ -1,0 +1,623 @@
+// fp32 convolution (+ Affine, Relu) and the 3x3 stride-2 pad-1 MaxPool behind it in one pass: the stem of a
+// Bi-Real-style net (dabnn/fconv.h:14-76, dabnn/layers/Affine.cpp:10-23, dabnn/layers/MaxPool.cpp:209-246).  The
+// convolution's output -- four times the size of the pooled tensor -- never goes to memory.
+//
+// A 512-thread block owns a band of R whole rows of the convolution's output of one image, R * OW = 448 pixels, and
+// 64 output channels.  It multiplies like the plain float convolution (implicit GEMM, rows = pixels, depth = (kh, kw,
+// c), two LDS buffers of SK-deep slices, v_mfma_f32_16x16x4_f32; eight waves as 4 x 2, a wave holds 112 pixels x 32
+// channels), leaves the band in LDS and pools it there.  A pooled row 2*py-1 .. 2*py+1 lies inside the band for all
+// but the band's first pooled row, which also needs the last row of the band above: every block writes the
+// horizontal maxima of its last row to a carry buffer, and a second, small kernel folds the carry of the band above
+// into the first pooled row of each band (a maximum does not depend on the order of its operands).  With the pooled
+// tensor the kernels can write its sign bits, the packed input of the binary convolution that follows
+// (dabnn/bitpack.h:277-293).
+#include <float.h>
+
+#include <type_traits>
+
+#include "common.h"
+
+namespace dab {
+
+struct FconvPoolArgs {
+    const float *x;
+    const float *w;
+    const float *bias;
+    const float *aff_a;
+    const float *aff_b;
+    float *pooled;    // [n][ph][pw][cout]
+    float *carry;     // [n][bands][pw][cout]
+    uint64_t *bits;   // [n][ph][pw][cout/64] or null
+    int n, h, wd, c;
+    int kw, dil_h, dil_w;
+    int pad_h, pad_w, stride_h, stride_w;
+    int oh, ow, cout;
+    int K;  // kh*kw*c
+    int relu;
+    int band_rows, bands;  // R, bands per image
+    int ph, pw;
+    int ytiles;  // 64-channel tiles of cout
+    FastDiv div_ow, div_c, div_kw, div_bands, div_ytiles;
+};
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t kPoolOob = 0x80000000u;  // beyond every descriptor used here (all shorter than 2^30 bytes)
+constexpr int kBandPixels = 448, kBandChannels = 64, kBandThreads = 512;
+constexpr int kStageStride = 68;  // floats per pixel row of the staged band: the 64 lanes of a store hit 64 banks
+
+template <int CV>
+struct BandSlice {
+    static constexpr int depth = CV == 3 ? 24 : 32;  // eight taps of three channels / eight groups of four channels
+    static constexpr int stride = depth + 4;         // LDS row stride in floats
+    static constexpr int loop_floats = 2 * (kBandPixels + kBandChannels) * stride;
+    static constexpr int stage_floats = kBandPixels * kStageStride;
+    static constexpr int lds_floats = loop_floats > stage_floats ? loop_floats : stage_floats;
+};
+
+// max of three values as the reference's loop computes it for results of arithmetic (v > m ? v : m skips a NaN; a
+// convolution's result is never a signalling NaN, the only kind the instruction treats differently)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float4 max3(float4 a, float4 b, float4 c) {
+    return make_float4(max3(a.x, b.x, c.x), max3(a.y, b.y, c.y), max3(a.z, b.z, c.z), max3(a.w, b.w, c.w));
+}
+
+// What the epilogue needs to know of a finished band.
+struct BandOut {
+    int img, band, row0, n0, ytile;
+};
+
+// A finished band (a wave's accumulators: 7 x 2 tiles of 16 pixels x 16 channels, wave (wm, wn) = pixels 112*wm ..,
+// channels 32*wn ..) goes through LDS to the pooled tensor, the carry and the sign bits.  All threads of the block
+// call it after a barrier that ended every other use of `stage`.
+template <bool SIGN>
+__device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *stage, const f32x4v (&acc)[7][2], const BandOut o,
+                                              int tid, int wm, int wn, int f_s, int f_i) {
+    constexpr int TM = 7, TN = 2;
+    // The band goes to LDS (the slices are dead: the loop ended with a barrier): + bias, Affine (a*v + b, two
+    // roundings), Relu, in the reference's order.  Accumulator element e of lane l: pixel 4*(l/16) + e, channel l % 16.
+    auto stage_all = [&](auto has_bias, auto has_affine, auto has_relu) {
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = wn * (TN * 16) + j * 16 + f_i, co = o.n0 + col;
+            const bool co_ok = co < p.cout;
+            const float bias = (decltype(has_bias)::value && co_ok) ? p.bias[co] : 0.f;
+            const float fa = (decltype(has_affine)::value && co_ok) ? p.aff_a[co] : 0.f;
+            const float fb = (decltype(has_affine)::value && co_ok) ? p.aff_b[co] : 0.f;
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float v = acc[i][j][e];
+                    if constexpr (decltype(has_bias)::value) v = v + bias;
+                    if constexpr (decltype(has_affine)::value) {
+                        const float prod = fa * v;
+                        v = prod + fb;
+                    }
+                    if constexpr (decltype(has_relu)::value) v = v > 0.f ? v : 0.f;
+                    stage[(wm * (TM * 16) + i * 16 + 4 * f_s + e) * kStageStride + col] = v;
+                }
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    switch ((p.bias ? 4 : 0) | (p.aff_a ? 2 : 0) | (p.relu ? 1 : 0)) {
+        case 0: stage_all(F{}, F{}, F{}); break;
+        case 1: stage_all(F{}, F{}, T{}); break;
+        case 2: stage_all(F{}, T{}, F{}); break;
+        case 3: stage_all(F{}, T{}, T{}); break;
+        case 4: stage_all(T{}, F{}, F{}); break;
+        case 5: stage_all(T{}, F{}, T{}); break;
+        case 6: stage_all(T{}, T{}, F{}); break;
+        default: stage_all(T{}, T{}, T{}); break;
+    }
+    __syncthreads();
+
+    // Pooling: a thread takes four channels of one pooled column and walks down the band's rows.  h = the maximum
+    // of the row's three columns 2*px-1 .. 2*px+1 (the first pooled column has two; one is read twice).  Pooled
+    // row q is max(h[2q-1], h[2q], h[2q+1]); for q = 0 the row above the band is left out: row -1 of the image
+    // does not exist, and the last row of the band above arrives through the carry, which is this band's h[R-1].
+    for (int it = tid; it < p.pw * 16; it += kBandThreads) {
+        const int c4 = it & 15, px = it >> 4;
+        const int co = o.n0 + c4 * 4;
+        const float *col0 = &stage[(px == 0 ? 0 : 2 * px - 1) * kStageStride + c4 * 4];
+        const float *col1 = &stage[(2 * px) * kStageStride + c4 * 4];
+        const float4 lowest = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+        float4 prev = lowest, even = lowest;
+        for (int r = 0; r < p.band_rows; ++r) {
+            const int ro = r * p.ow * kStageStride;
+            const float4 h = max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
+                                  *reinterpret_cast<const float4 *>(col1 + ro + kStageStride));
+            if (r & 1) {
+                const float4 m = max3(even, h, lowest);
+                if (co < p.cout) {
+                    const size_t pix = (size_t)(o.img * p.ph + ((o.row0 + r) >> 1)) * p.pw + px;
+                    *reinterpret_cast<float4 *>(p.pooled + pix * p.cout + co) = m;
+                    if constexpr (SIGN) {
+                        // cout % 64 == 0: the 16 lanes of a pixel are one row of lanes, all of them here
+                        const uint32_t nib = sign_nibble(m);
+                        uint32_t lo = c4 < 8 ? nib << (4 * c4) : 0u, hi = c4 >= 8 ? nib << (4 * (c4 - 8)) : 0u;
+                        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+                        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+                        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+                        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+                        if (c4 == 0) p.bits[pix * (p.cout >> 6) + o.ytile] = ((uint64_t)hi << 32) | lo;
+                    }
+                }
+            } else {
+                even = max3(prev, h, lowest);  // r == 0: prev is the lowest value, the row above is left out
+            }
+            prev = h;
+        }
+        if (co < p.cout) {
+            const float4 m = max3(prev, lowest, lowest);
+            *reinterpret_cast<float4 *>(p.carry + ((size_t)(o.img * p.bands + o.band) * p.pw + px) * p.cout + co) = m;
+        }
+    }
+}
+
+template <int CV, bool SIGN>
+__global__ __launch_bounds__(kBandThreads) void fconv_maxpool_kernel(const FconvPoolArgs p) {
+    constexpr int BM = kBandPixels, BN = kBandChannels;
+    constexpr int SK = BandSlice<CV>::depth, RS = BandSlice<CV>::stride;
+    constexpr int LK = SK / CV;              // loader lanes along the depth
+    constexpr int RP = kBandThreads / LK;    // tile rows fetched per pass of the block
+    constexpr int APT = BM / RP;             // pixel rows per thread and slice
+    constexpr int TM = 7, TN = 2;            // 16 x 16 matrix-core tiles per wave
+    static_assert(LK == 8 && RP == 64 && APT == 7 && RP == BN, "loader shape");
+    __shared__ __attribute__((aligned(16))) float smem[BandSlice<CV>::lds_floats];
+    auto As = [&](int buf, int row, int k) -> float & { return smem[(buf * (BM + BN) + row) * RS + k]; };
+    auto Bs = [&](int buf, int row, int k) -> float & { return smem[(buf * (BM + BN) + BM + row) * RS + k]; };
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l_k = tid % LK, l_r = tid / LK;  // loader: depth group l_k of the slice, tile rows l_r + RP*i
+    const uint32_t img_bytes = (uint32_t)(p.h * p.wd * p.c) * 4u;
+    const uint32_t b_row = (uint32_t)l_r * p.K * 4u;
+
+    // the band of the loader (the one whose slices are being fetched) and its addresses
+    int img, band, row0, n0, rows_n;
+    __amdgpu_buffer_rsrc_t x_rsrc, w_rsrc;
+    uint32_t a_base[APT];  // byte offset of (y0, x0, channel 0) in the image, modulo 2^32
+    int a_x0[APT];
+    int a_lr[APT], a_ox[APT];  // the thread's pixels inside a band, the same for every band
+#pragma unroll
+    for (int i = 0; i < APT; ++i) {
+        const int r = l_r + RP * i;
+        a_lr[i] = (int)p.div_ow.div((uint32_t)r), a_ox[i] = r - a_lr[i] * p.ow;
+    }
+    auto enter = [&](int item) {
+        const int bi = (int)p.div_ytiles.div((uint32_t)item);
+        n0 = (item - bi * p.ytiles) * BN;
+        img = (int)p.div_bands.div((uint32_t)bi);
+        band = bi - img * p.bands;
+        row0 = band * p.band_rows;
+        // The descriptor covers one image: a tap above or below the image has an offset that is negative modulo
+        // 2^32 or at least the image's size, and reads as zero without a test; only the column needs one.
+        x_rsrc = make_rsrc(p.x + (size_t)img * p.h * p.wd * p.c, img_bytes);
+        rows_n = p.cout - n0 < BN ? p.cout - n0 : BN;
+        w_rsrc = make_rsrc(p.w + (size_t)n0 * p.K, (uint32_t)rows_n * p.K * 4u);
+#pragma unroll
+        for (int i = 0; i < APT; ++i) {
+            const int y0 = (row0 + a_lr[i]) * p.stride_h - p.pad_h, x0 = a_ox[i] * p.stride_w - p.pad_w;
+            a_base[i] = (uint32_t)((y0 * p.wd + x0) * p.c) * 4u;
+            a_x0[i] = x0;
+        }
+    };
+
+    typedef float f32xcv __attribute__((ext_vector_type(CV)));
+    f32xcv a_reg[APT], b_reg;
+    auto load_cv = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off) -> f32xcv {
+        // bit-cast as a whole: casting single elements of a vector buffer load makes the compiler shrink the load
+        if constexpr (CV == 3)
+            return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)off, 0, 0));
+        else
+            return __builtin_bit_cast(f32xcv, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    };
+    auto fetch = [&](int k0) {
+        // CV == 3: lane group = tap, channels 0..2 (c == 3).  CV == 4: four consecutive channels of a tap (c % 4 == 0).
+        const int k = k0 + CV * l_k;
+        const bool k_ok = k < p.K;
+        int tap, ch;
+        if constexpr (CV == 3) {
+            tap = (int)((uint32_t)k0 / 3u) + l_k, ch = 0;
+        } else {
+            tap = (int)p.div_c.div((uint32_t)k), ch = k - tap * p.c;
+        }
+        const int ty = (int)p.div_kw.div((uint32_t)tap), tx = tap - ty * p.kw;
+        const int dy = ty * p.dil_h, dx = tx * p.dil_w;
+        // a depth past the end: 2^31 added to an offset of magnitude below 2^30 stays out of range
+        const uint32_t delta = k_ok ? (uint32_t)((dy * p.wd + dx) * p.c + ch) * 4u : kPoolOob;
+#pragma unroll
+        for (int i = 0; i < APT; ++i)
+            a_reg[i] = load_cv(x_rsrc, (unsigned)(a_x0[i] + dx) < (unsigned)p.wd ? a_base[i] + delta : kPoolOob);
+        b_reg = load_cv(w_rsrc, (k_ok && l_r < rows_n) ? b_row + (uint32_t)k * 4u : kPoolOob);
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < APT; ++i)
+#pragma unroll
+            for (int c = 0; c < CV; ++c) As(buf, l_r + RP * i, l_k * CV + c) = a_reg[i][c];
+#pragma unroll
+        for (int c = 0; c < CV; ++c) Bs(buf, l_r, l_k * CV + c) = b_reg[c];
+    };
+
+    // operand lane l of the instruction: row / column l % 16, depth slot l / 16.  Which depth sits in which of the
+    // four slots does not matter as long as both operands agree: a lane reads two consecutive depths at once and
+    // uses them in two instructions.
+    const int f_s = lane >> 4, f_i = lane & 15;
+    const int n_items = p.n * p.bands * p.ytiles;
+    int item = blockIdx.x;
+    if (item >= n_items) return;
+    enter(item);
+    fetch(0);
+    for (;;) {
+        // here: the first slice of `item` is in registers, every thread is past its last read of the LDS
+        commit(0);
+        __syncthreads();
+        f32x4v acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+        int buf = 0;
+        for (int k0 = 0; k0 < p.K; k0 += SK, buf ^= 1) {
+            const bool more = k0 + SK < p.K;
+            if (more) fetch(k0 + SK);
+#pragma unroll
+            for (int g = 0; g < SK / 8; ++g) {
+                // the last slice may end early: groups that lie wholly past the depth hold zeros on both sides
+                if (g > 0 && k0 + g * 8 >= p.K) break;
+                const int kb = g * 8 + 2 * f_s;
+                float2 a2[TM], b2[TN];
+#pragma unroll
+                for (int i = 0; i < TM; ++i) a2[i] = *reinterpret_cast<const float2 *>(&As(buf, wm * (TM * 16) + i * 16 + f_i, kb));
+#pragma unroll
+                for (int j = 0; j < TN; ++j) b2[j] = *reinterpret_cast<const float2 *>(&Bs(buf, wn * (TN * 16) + j * 16 + f_i, kb));
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a2[i].x, b2[j].x, acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a2[i].y, b2[j].y, acc[i][j], 0, 0, 0);
+                    }
+            }
+            // the other buffer was last read before the barrier that ended the previous slice
+            if (more) commit(buf ^ 1);
+            __syncthreads();
+        }
+
+        // what the epilogue needs of this band, then the next band's first slice is asked for: its latency hides
+        // behind the epilogue
+        const int e_img = img, e_band = band, e_row0 = row0, e_n0 = n0;
+        const int next = item + gridDim.x;
+        const bool has_next = next < n_items;
+        if (has_next) {
+            enter(next);
+            fetch(0);
+        }
+
+        band_epilogue<SIGN>(p, smem, acc, BandOut{e_img, e_band, e_row0, e_n0, e_n0 / BN}, tid, wm, wn, f_s, f_i);
+        if (!has_next) break;
+        item = next;
+        __syncthreads();  // the staged band is dead
+    }
+}
+
+// The ImageNet stem itself -- 7x7, stride 2, pad 3 on three-channel images whose output is 112 pixels wide -- without
+// an im2col stage: a band's 13 input rows go to LDS as they are (229 pixels from x = -3, zeros outside the image), and
+// the matrix-core operands are read straight from them.  Wave (wm, wn) owns output row wm of the band and 32
+// channels; an output pixel's 21 values of one kernel row are contiguous (tile floats 6*ox + k', k' = 3*tx + ch),
+// so for every kernel row a lane's operand addresses are one base plus constants: depth slot s of the instruction
+// takes k' = 4s .. 4s+3 in four instructions, then k' = 16 + s in a fifth, and the seven k' = 20 of all kernel rows
+// fill two more (slot s = kernel row s, then 4 + s; the eighth slot's weight is zero).  148 depths for 147.  The
+// block's 64 filters sit in LDS in that order for all of its bands; the next band's rows are fetched into registers
+// while the current one is multiplied.
+constexpr int kTileStride = 688;                    // floats per tile row: 229 pixels x 3, rounded up to even
+constexpr int kTileRows = 13, kTilePixels = 229;
+constexpr int kFilterStride = 148;                  // 7 x (16 + 4) + 7 + 1 floats per filter
+constexpr int kFilterFloats = kBandChannels * kFilterStride;
+constexpr int kStemLdsFloats = kFilterFloats + kBandPixels * kStageStride;  // the tile shares the staged band's space
+constexpr int kTileLoads = (kTileRows * kTilePixels + kBandThreads - 1) / kBandThreads;
+
+template <bool SIGN>
+__global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const FconvPoolArgs p) {
+    constexpr int BN = kBandChannels, TM = 7, TN = 2;
+    static_assert(kTileStride * kTileRows <= kBandPixels * kStageStride, "the tile fits the staged band's space");
+    __shared__ __attribute__((aligned(16))) float smem[kStemLdsFloats];
+    float *const wl = smem, *const tile = smem + kFilterFloats;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int f_s = lane >> 4, f_i = lane & 15;
+    const uint32_t img_bytes = (uint32_t)(p.h * p.wd * 3) * 4u;
+    const int n_items = p.n * p.bands * p.ytiles;
+    int item = blockIdx.x;
+    if (item >= n_items) return;
+
+    // the thread's pixels of a tile: byte offset from the tile's first row in the image, and place in LDS
+    uint32_t t_off[kTileLoads];
+    int t_lds[kTileLoads];
+#pragma unroll
+    for (int j = 0; j < kTileLoads; ++j) {
+        const int q = tid + kBandThreads * j;
+        const int ry = q / kTilePixels, cx = q - ry * kTilePixels, x = cx - 3;
+        const bool ok = q < kTileRows * kTilePixels && (unsigned)x < (unsigned)p.wd;
+        t_off[j] = ok ? (uint32_t)((ry * p.wd + x) * 12) : kPoolOob;
+        t_lds[j] = q < kTileRows * kTilePixels ? ry * kTileStride + cx * 3 : -1;
+    }
+    typedef float f32x3v __attribute__((ext_vector_type(3)));
+    f32x3v pf[kTileLoads];
+    int img, band, row0, n0;
+    auto enter = [&](int it) {
+        const int bi = (int)p.div_ytiles.div((uint32_t)it);
+        n0 = (it - bi * p.ytiles) * BN;
+        img = (int)p.div_bands.div((uint32_t)bi);
+        band = bi - img * p.bands;
+        row0 = band * 4;
+    };
+    auto fetch_tile = [&]() {
+        // One descriptor per image: rows above and below it have offsets that are negative modulo 2^32 or at least
+        // the image's size, and read as zero; columns outside carry kPoolOob, which stays out of range after the
+        // addition of a row offset of magnitude below 2^30.
+        const auto x_rsrc = make_rsrc(p.x + (size_t)img * p.h * p.wd * 3, img_bytes);
+        const uint32_t base = (uint32_t)((2 * row0 - 3) * p.wd * 12);
+#pragma unroll
+        for (int j = 0; j < kTileLoads; ++j)
+            pf[j] = __builtin_bit_cast(f32x3v, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, (int)(base + t_off[j]), 0, 0));
+    };
+
+    // lane constants of the operand reads (floats)
+    const int a_row = 2 * wm * kTileStride + 6 * f_i;
+    const float *pa = tile + a_row + 4 * f_s, *pa4 = tile + a_row + 16 + f_s;
+    const float *pa_l0 = tile + a_row + f_s * kTileStride + 20;
+    const float *pa_l1 = tile + a_row + (f_s < 3 ? 4 + f_s : 6) * kTileStride + 20;
+    const float *pb = wl + (wn * 32 + f_i) * kFilterStride + 4 * f_s, *pb4 = pb + 16 - 3 * f_s;
+    const float *pb_l = wl + (wn * 32 + f_i) * kFilterStride + 140 + f_s;
+
+    enter(item);
+    fetch_tile();
+    int filters_of = -1;  // the channel tile whose filters are in LDS
+    for (;;) {
+        // here: the band's rows are in registers (or on their way), every thread is past its last read of the LDS
+        if (n0 != filters_of) {
+            filters_of = n0;
+            const int rows_n = p.cout - n0 < BN ? p.cout - n0 : BN;
+            for (int idx = tid; idx < kFilterFloats; idx += kBandThreads) {
+                const int co = idx / kFilterStride, r = idx - co * kFilterStride;
+                // r < 140: kernel row r / 20, k' = r % 20; then k' = 20 of kernel rows 0..6; the last float is zero
+                const int k = r < 140 ? (r / 20) * 21 + r % 20 : (r - 140) * 21 + 20;
+                wl[idx] = (co < rows_n && r < 147) ? p.w[(size_t)(n0 + co) * 147 + k] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kTileLoads; ++j)
+            if (t_lds[j] >= 0) {
+                tile[t_lds[j]] = pf[j][0], tile[t_lds[j] + 1] = pf[j][1], tile[t_lds[j] + 2] = pf[j][2];
+            }
+        __syncthreads();
+
+        const BandOut o{img, band, row0, n0, n0 / BN};
+        const int next = item + gridDim.x;
+        const bool has_next = next < n_items;
+        if (has_next) {
+            enter(next);
+            fetch_tile();
+        }
+
+        f32x4v acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ty = 0; ty < 7; ++ty) {
+            float2 alo[TM], ahi[TM];
+            float a4[TM];
+            float4 b[TN];
+            float b4[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                alo[i] = *reinterpret_cast<const float2 *>(pa + ty * kTileStride + 96 * i);
+                ahi[i] = *reinterpret_cast<const float2 *>(pa + ty * kTileStride + 96 * i + 2);
+                a4[i] = pa4[ty * kTileStride + 96 * i];
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                b[j] = *reinterpret_cast<const float4 *>(pb + ty * 20 + j * 16 * kFilterStride);
+                b4[j] = pb4[ty * 20 + j * 16 * kFilterStride];
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(alo[i].x, b[j].x, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(alo[i].y, b[j].y, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ahi[i].x, b[j].z, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ahi[i].y, b[j].w, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[i], b4[j], acc[i][j], 0, 0, 0);
+                }
+        }
+        {
+            float al0[TM], al1[TM], bl0[TN], bl1[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) al0[i] = pa_l0[96 * i], al1[i] = pa_l1[96 * i];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bl0[j] = pb_l[j * 16 * kFilterStride], bl1[j] = pb_l[4 + j * 16 * kFilterStride];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(al0[i], bl0[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(al1[i], bl1[j], acc[i][j], 0, 0, 0);
+                }
+        }
+        __syncthreads();  // the tile is dead: the staged band takes its place
+        band_epilogue<SIGN>(p, tile, acc, o, tid, wm, wn, f_s, f_i);
+        if (!has_next) break;
+        item = next;
+        __syncthreads();  // the staged band is dead
+    }
+}
+
+struct CarryArgs {
+    float4 *pooled;
+    const float4 *carry;
+    uint64_t *bits;
+    uint32_t total;  // n * (bands - 1) * pw * c4
+    int bands, ph, pw, c4, half;
+    FastDiv div_c4, div_pw, div_bm1;
+};
+
+// pooled[first row of band b] = max(itself, carry of band b - 1), b >= 1; SIGN: and that row's sign bits again.
+template <bool SIGN>
+__global__ __launch_bounds__(256) void maxpool_carry_kernel(const CarryArgs p) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= p.total) return;
+    uint32_t t = p.div_c4.div(idx);
+    const int ch = (int)(idx - t * p.c4);
+    uint32_t t2 = p.div_pw.div(t);
+    const int px = (int)(t - t2 * p.pw);
+    const uint32_t img = p.div_bm1.div(t2);
+    const int b = (int)(t2 - img * (p.bands - 1)) + 1;
+    const size_t pix = ((size_t)img * p.ph + (size_t)b * p.half) * p.pw + px;
+    const float4 m = p.pooled[pix * p.c4 + ch];
+    const float4 v = p.carry[(((size_t)img * p.bands + (b - 1)) * p.pw + px) * p.c4 + ch];
+    float4 r;
+    r.x = v.x > m.x ? v.x : m.x, r.y = v.y > m.y ? v.y : m.y, r.z = v.z > m.z ? v.z : m.z, r.w = v.w > m.w ? v.w : m.w;
+    p.pooled[pix * p.c4 + ch] = r;
+    if constexpr (SIGN) {
+        // c4 % 16 == 0 and total % 16 == 0: a row of lanes is one word's channels, complete or returned as a whole
+        const int part = ch & 15;
+        const uint32_t nib = sign_nibble(r);
+        uint32_t lo = part < 8 ? nib << (4 * part) : 0u, hi = part >= 8 ? nib << (4 * (part - 8)) : 0u;
+        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+        if (part == 0) p.bits[(pix * p.c4 + ch) >> 4] = ((uint64_t)hi << 32) | lo;
+    }
+}
+
+// Geometry of the fused pass, or false when the shapes do not fit it.
+struct BandPlan {
+    int oh, ow, band_rows, bands, ph, pw;
+};
+static bool plan_bands(int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
+                       int dil_w, int cout, BandPlan &b) {
+    if (h <= 0 || w <= 0 || c <= 0 || kh <= 0 || kw <= 0 || pad_h < 0 || pad_w < 0 || stride_h <= 0 || stride_w <= 0 ||
+        dil_h <= 0 || dil_w <= 0 || cout <= 0)
+        return false;
+    b.oh = out_dim(h, pad_h, kh, dil_h, stride_h), b.ow = out_dim(w, pad_w, kw, dil_w, stride_w);
+    if (b.oh <= 0 || b.ow <= 0 || kBandPixels % b.ow != 0) return false;
+    b.band_rows = kBandPixels / b.ow;
+    if (b.band_rows % 2 != 0 || b.ow % 2 != 0 || b.oh % b.band_rows != 0) return false;
+    b.bands = b.oh / b.band_rows;
+    b.ph = b.oh / 2, b.pw = b.ow / 2;  // out_dim(oh, 1, 3, 1, 2) for even oh
+    if (cout % 4 != 0 || !(c == 3 || c % 4 == 0)) return false;
+    // one image, 64 filters and 64 output pixels' worth of offsets stay below 2^30 bytes
+    if (((long long)h + (long long)kh * dil_h + pad_h) * w * c * 4 >= (1ll << 30) || 64ll * kh * kw * c * 4 >= (1ll << 30)) return false;
+    return true;
+}
+
+}  // namespace dab
+
+extern "C" int64_t dab_fconv_maxpool_carry_floats(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                                                  int stride_h, int stride_w, int dil_h, int dil_w, int cout) {
+    dab::BandPlan b;
+    if (n <= 0 || !dab::plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b)) return 0;
+    return (int64_t)n * b.bands * b.pw * cout;
+}
+
+extern "C" int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
+                                      int stride_w, int dil_h, int dil_w, int cout) {
+    dab::BandPlan b;
+    if (n <= 0 || !dab::plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b)) return 0;
+    // a band is a long work item and a CU holds one block: below several rounds of blocks the last round's idle CUs
+    // cost more than the saved traffic
+    const long long blocks = (long long)n * b.bands * ((cout + dab::kBandChannels - 1) / dab::kBandChannels);
+    return blocks >= 4ll * (dab::simd_count() / 4) ? 1 : 0;
+}
+
+extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                 const float *aff_a, const float *aff_b, int relu, int kh, int kw, int pad_h, int pad_w,
+                                 int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *pooled,
+                                 uint64_t *pooled_packed, float *carry, dab_stream_t stream) {
+    using namespace dab;
+    const char *fn = "dab_fconv_maxpool";
+    DAB_REQUIRE(x && wgt && pooled && carry, "%s: null pointer", fn);
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && kh > 0 && kw > 0 && cout > 0, "%s: non-positive dimension", fn);
+    DAB_REQUIRE(pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0,
+                "%s: bad pad/stride/dilation", fn);
+    DAB_REQUIRE((aff_a == nullptr) == (aff_b == nullptr), "%s: affine needs both coefficient vectors", fn);
+    BandPlan b;
+    if (!plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b))
+        return fail(DAB_EUNSUPPORTED,
+                    "%s: needs an output width that divides 448 into an even number of rows, an output height that is a "
+                    "multiple of it, 3 or a multiple of 4 input channels and cout %% 4 == 0 (got %dx%dx%d -> %dx%dx%d)",
+                    fn, h, w, c, out_dim(h, pad_h, kh, dil_h, stride_h), out_dim(w, pad_w, kw, dil_w, stride_w), cout);
+    if (pooled_packed && cout % 64 != 0) return fail(DAB_EUNSUPPORTED, "%s: sign bits need cout %% 64 == 0", fn);
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt) | reinterpret_cast<uintptr_t>(pooled) |
+         reinterpret_cast<uintptr_t>(carry)) % 16 != 0)
+        return fail(DAB_EUNSUPPORTED, "%s: needs 16-byte aligned buffers", fn);
+    const long long pooled_elems = (long long)n * b.ph * b.pw * cout;
+    if ((long long)n * b.oh >= (1ll << 31) || pooled_elems >= (1ll << 33))
+        return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
+    FconvPoolArgs a;
+    a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.relu = relu;
+    a.pooled = pooled, a.carry = carry, a.bits = pooled_packed;
+    a.n = n, a.h = h, a.wd = w, a.c = c;
+    a.kw = kw, a.dil_h = dil_h, a.dil_w = dil_w;
+    a.pad_h = pad_h, a.pad_w = pad_w, a.stride_h = stride_h, a.stride_w = stride_w;
+    a.oh = b.oh, a.ow = b.ow, a.cout = cout, a.K = kh * kw * c;
+    a.band_rows = b.band_rows, a.bands = b.bands, a.ph = b.ph, a.pw = b.pw;
+    a.div_ow = FastDiv((uint32_t)b.ow), a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv((uint32_t)kw);
+    a.ytiles = (cout + kBandChannels - 1) / kBandChannels;
+    a.div_bands = FastDiv((uint32_t)b.bands), a.div_ytiles = FastDiv((uint32_t)a.ytiles);
+    hipStream_t s = as_stream(stream);
+    // one block per CU (its LDS holds one), each walking through the work items gridDim.x apart
+    const long long items = (long long)n * b.bands * a.ytiles;
+    if (items >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
+    const int cus = simd_count() / 4;
+    const dim3 grid((unsigned)(items < cus ? items : cus));
+    if (c == 3 && kh == 7 && kw == 7 && stride_h == 2 && stride_w == 2 && pad_h == 3 && pad_w == 3 && dil_h == 1 &&
+        dil_w == 1 && b.ow == 112) {
+        if (pooled_packed)
+            hipLaunchKernelGGL(fconv7x7s2_maxpool_kernel<true>, grid, dim3(kBandThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL(fconv7x7s2_maxpool_kernel<false>, grid, dim3(kBandThreads), 0, s, a);
+    } else if (c == 3) {
+        if (pooled_packed)
+            hipLaunchKernelGGL((fconv_maxpool_kernel<3, true>), grid, dim3(kBandThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((fconv_maxpool_kernel<3, false>), grid, dim3(kBandThreads), 0, s, a);
+    } else {
+        if (pooled_packed)
+            hipLaunchKernelGGL((fconv_maxpool_kernel<4, true>), grid, dim3(kBandThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((fconv_maxpool_kernel<4, false>), grid, dim3(kBandThreads), 0, s, a);
+    }
+    DAB_LAUNCH_CHECK();
+    if (b.bands > 1) {
+        CarryArgs ca;
+        ca.pooled = reinterpret_cast<float4 *>(pooled), ca.carry = reinterpret_cast<const float4 *>(carry);
+        ca.bits = pooled_packed;
+        ca.bands = b.bands, ca.ph = b.ph, ca.pw = b.pw, ca.c4 = cout / 4, ca.half = b.band_rows / 2;
+        const long long total = (long long)n * (b.bands - 1) * b.pw * ca.c4;
+        if (total >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
+        ca.total = (uint32_t)total;
+        ca.div_c4 = FastDiv((uint32_t)ca.c4), ca.div_pw = FastDiv((uint32_t)b.pw), ca.div_bm1 = FastDiv((uint32_t)(b.bands - 1));
+        const unsigned blocks = (unsigned)((total + 255) / 256);
+        if (pooled_packed)
+            hipLaunchKernelGGL(maxpool_carry_kernel<true>, dim3(blocks), dim3(256), 0, s, ca);
+        else
+            hipLaunchKernelGGL(maxpool_carry_kernel<false>, dim3(blocks), dim3(256), 0, s, ca);
+        DAB_LAUNCH_CHECK();
+    }
+    return DAB_OK;
+}

@@ -237,6 +237,8 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
         if (more) fetch(k0 + SK);
 #pragma unroll
         for (int g = 0; g < WK / 8; ++g) {  // this wave's depths of the slice, 8 at a time
+            // the last slice may end early: groups that lie wholly past the depth hold zeros on both sides
+            if (KSPLIT == 1 && g > 0 && k0 + g * 8 >= p.K) break;
             const int kb = ks * WK + g * 8 + f_k * 4;
             float4 a4[TM], b4[TN];
 #pragma unroll

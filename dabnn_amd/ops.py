@@ -262,6 +262,39 @@ def ave_pool2_fconv1x1(x, weight, bias, a, b, relu):
     return pooled, out
 
 
+def fconv_maxpool(x, weight, bias, a, b, relu, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h=1, dil_w=1, want_sign=False):
+    """FpConv2D (+ Affine + Relu) and MaxPool 3x3 stride 2 pad 1 in one pass; returns (pooled, pack_mat of it or None)."""
+    _need(x, torch.float32, "x")
+    _need(weight, torch.float32, "weight")
+    n, h, w, c = x.shape
+    cout = weight.shape[0]
+    if weight.numel() != cout * kh * kw * c:
+        raise capi.DabError(capi.DAB_EINVAL, "fconv_maxpool: weight must be [cout, kh, kw, c]")
+    def opt(t, name):
+        if t is None:
+            return None
+        _need(t, torch.float32, name)
+        if t.numel() != cout:
+            raise capi.DabError(capi.DAB_EINVAL, "fconv_maxpool: %s does not match the channel count" % name)
+        return _ptr(t)
+    geom = (n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout)
+    carry_floats = lib.dab_fconv_maxpool_carry_floats(*geom)
+    oh, ow = out_dim(h, pad_h, kh, stride_h, dil_h), out_dim(w, pad_w, kw, stride_w, dil_w)
+    ph, pw = max(oh, 0) // 2, max(ow, 0) // 2
+    pooled = _empty((n, ph, pw, cout), torch.float32, x.device)
+    carry = _empty((max(int(carry_floats), 4),), torch.float32, x.device)
+    packed = _empty((n, ph, pw, max(cout // 64, 1)), torch.int64, x.device) if want_sign else None
+    check(lib.dab_fconv_maxpool(_ptr(x), n, h, w, c, _ptr(weight), opt(bias, "bias"), opt(a, "a"), opt(b, "b"),
+                                int(bool(relu)), kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout,
+                                _ptr(pooled), _ptr(packed) if want_sign else None, _ptr(carry), _stream()))
+    return pooled, packed
+
+
+def fconv_maxpool_pays(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout):
+    """Whether the one-pass convolution + MaxPool takes these shapes and beats the two launches on this device."""
+    return bool(lib.dab_fconv_maxpool_pays(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout))
+
+
 def affine_inplace(x, a, b):
     """affine_inplace (dabnn/layers/Affine.cpp:10-23)."""
     _need(x, torch.float32, "x")

@@ -193,6 +193,27 @@ DAB_API int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, c
                                    const float *a, const float *b, int relu, int cout, float *pooled, float *out,
                                    dab_stream_t stream);
 
+/*
+ * FpConv2D (dabnn/fconv.h:14-76) with the optional Affine and Relu of dab_fconv_affine_relu, followed by MaxPool 3x3,
+ * stride 2, pad 1 (max_pool_fallback, dabnn/layers/MaxPool.cpp:209-246), in one pass that never writes the
+ * convolution's output: the stem of a Bi-Real-style net.  pooled [n][oh/2][ow/2][cout] receives what dab_max_pool
+ * computes from the convolution's result; pooled_packed, when not null (cout % 64 == 0), pack_mat of it
+ * (dabnn/bitpack.h:277-293) as dab_max_pool_sign writes it.  carry is a workspace of
+ * dab_fconv_maxpool_carry_floats(...) floats.  Shapes: the convolution's output width ow must divide 448 into an even
+ * number of rows (28, 56, 112 or 224), oh must be a multiple of 448/ow, c must be 3 or a multiple of 4, cout a
+ * multiple of 4, all buffers 16-byte aligned (DAB_EUNSUPPORTED otherwise).
+ * dab_fconv_maxpool_carry_floats returns 0 for shapes the pass does not take; dab_fconv_maxpool_pays returns 1 when
+ * the problem is also large enough on the current device for the pass to beat dab_fconv_affine_relu + dab_max_pool_sign.
+ */
+DAB_API int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                              const float *a, const float *b, int relu, int kh, int kw, int pad_h, int pad_w,
+                              int stride_h, int stride_w, int dil_h, int dil_w, int cout, float *pooled,
+                              uint64_t *pooled_packed, float *carry, dab_stream_t stream);
+DAB_API int64_t dab_fconv_maxpool_carry_floats(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
+                                               int stride_h, int stride_w, int dil_h, int dil_w, int cout);
+DAB_API int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
+                                   int stride_w, int dil_h, int dil_w, int cout);
+
 /* affine_inplace (dabnn/layers/Affine.cpp:10-23): x[..., ch] = a[ch]*x[..., ch] + b[ch]. */
 DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, const float *b, dab_stream_t stream);
 

@@ -420,6 +420,76 @@ def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine)
         dab.ave_pool2_fconv1x1(dev_f(x[..., :3].copy()), dev_f(wgt[..., :3].copy()), None, None, None, False)
 
 
+@pytest.mark.parametrize("n,h,w,c,k,pad,stride,dil,cout,bias,affine,relu", [
+    # output width 28, 56, 112 (bands of 16, 8, 4 rows), one band per image and several, three-channel images and
+    # multiples of four channels, a depth that is no multiple of the slice, two channel tiles, a ragged channel tile
+    (2, 64, 56, 3, 7, 3, 2, 1, 64, False, True, False), (3, 16, 112, 3, 7, 3, 2, 1, 64, True, False, True),
+    (1, 224, 224, 3, 7, 3, 2, 1, 64, False, True, False), (2, 32, 56, 32, 3, 1, 1, 1, 64, False, True, True),
+    (2, 16, 28, 8, 3, 1, 1, 1, 128, True, True, False), (1, 16, 28, 4, 5, 2, 1, 1, 20, False, False, False),
+    (1, 36, 60, 3, 3, 0, 1, 2, 64, True, True, True),
+    # the 7x7 stride-2 stem at output width 112 has a kernel of its own: odd image sizes, two channel tiles on one
+    # block, a ragged channel tile, a single band
+    (2, 31, 223, 3, 7, 3, 2, 1, 128, True, True, True), (1, 8, 224, 3, 7, 3, 2, 1, 20, False, False, False),
+])
+def test_fconv_maxpool_one_pass(dab, n, h, w, c, k, pad, stride, dil, cout, bias, affine, relu):
+    """FpConv2D (+ Affine + Relu) + MaxPool 3x3 stride 2 pad 1 without the convolution's output in memory: within
+    the float tolerance of the CPU layers, bit for bit what max_pool makes of the separate float convolution on
+    the device when the data make fp32 sums exact, and the packed copy is pack_mat of the pooled tensor it wrote."""
+    r = rng(47)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    wgt = (r.standard_normal((cout, k, k, c)) / np.sqrt(k * k * c)).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32) if bias else None
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    sign = cout % 64 == 0
+
+    def cpu(x, wgt, bv, a, b):
+        out = []
+        for img in x:
+            y = orc.fconv(img, wgt, bv, k, k, pad, pad, stride, stride, dil, dil)
+            if affine:
+                y = orc.affine_inplace(y.copy(), a, b)
+            if relu:
+                y = np.maximum(y, 0)
+            out.append(orc.max_pool(y, 3, 3, 1, 1, 2, 2))
+        return np.stack(out)
+
+    def gpu(x, wgt, bv, a, b):
+        return dab.fconv_maxpool(dev_f(x), dev_f(wgt), dev_f(bv) if bias else None, dev_f(a) if affine else None,
+                                 dev_f(b) if affine else None, relu, k, k, pad, pad, stride, stride, dil, dil, want_sign=sign)
+
+    pooled, packed = gpu(x, wgt, bv, a, b)
+    got, want = pooled.cpu().numpy(), cpu(x, wgt, bv, a, b)
+    assert got.shape == want.shape
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * np.abs(want).max())
+    if sign:
+        np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in got]))
+    # small integers: every product and partial sum is exact in fp32, whatever the order of the additions
+    xi = r.integers(-3, 4, x.shape).astype(np.float32)
+    wi = r.integers(-2, 3, wgt.shape).astype(np.float32)
+    bi = r.integers(-5, 6, cout).astype(np.float32) if bias else None
+    ai, ci = r.integers(-2, 3, cout).astype(np.float32), r.integers(-9, 10, cout).astype(np.float32)
+    pooled, packed = gpu(xi, wi, bi, ai, ci)
+    want = cpu(xi, wi, bi, ai, ci)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want)
+    if sign:
+        np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+    sep = dab.fconv_affine_relu(dev_f(xi), dev_f(wi), dev_f(bi) if bias else None, dev_f(ai) if affine else None,
+                                dev_f(ci) if affine else None, relu, k, k, pad, pad, stride, stride, dil, dil)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), dab.max_pool(sep, 3, 3, 1, 1, 2, 2).cpu().numpy())
+
+
+def test_fconv_maxpool_rejects_other_shapes(dab):
+    x = torch.zeros((1, 60, 60, 3), device="cuda")
+    wgt = torch.zeros((64, 7, 7, 3), device="cuda")
+    with pytest.raises(RuntimeError, match="output width"):
+        dab.fconv_maxpool(x, wgt, None, None, None, False, 7, 7, 3, 3, 2, 2)  # 30 x 30 output
+    with pytest.raises(RuntimeError, match="output width"):
+        dab.fconv_maxpool(torch.zeros((1, 58, 56, 3), device="cuda"), wgt, None, None, None, False, 7, 7, 3, 3, 2, 2)  # 29 rows
+    with pytest.raises(RuntimeError, match="sign bits"):
+        dab.fconv_maxpool(torch.zeros((1, 64, 56, 3), device="cuda"), torch.zeros((32, 7, 7, 3), device="cuda"), None, None,
+                          None, False, 7, 7, 3, 3, 2, 2, want_sign=True)
+
+
 @pytest.mark.parametrize("shape", [(2, 5, 7, 64), (1, 3, 3, 5), (3, 16, 16, 192), (1, 1, 1, 1)])
 def test_prelu_bit_exact(dab, shape):
     r = rng(44)
