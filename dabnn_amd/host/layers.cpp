@@ -171,6 +171,17 @@ void FloatConv::forward_impl() const {
             static_cast<float *>(input_mat->data), static_cast<float *>(output_mat->data), stream()));
         return;
     }
+    if (fused_maxpool_out) {
+        dab_check(dab_fconv_maxpool(
+            static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
+            static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
+            fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
+            fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
+            pad_h, pad_w, stride_h, stride_w, dilation, dilation, weight_mat->n, static_cast<float *>(fused_maxpool_out->data),
+            fused_maxpool_sign ? static_cast<uint64_t *>(fused_maxpool_sign->data) : nullptr,
+            static_cast<float *>(fused_maxpool_carry->data), stream()));
+        return;
+    }
     dab_check(dab_fconv_affine_relu(
         static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
         static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
@@ -187,6 +198,7 @@ std::string FloatConv::to_str() const {
     if (fused_a) ss << " + Affine";
     if (fused_relu) ss << " + Relu";
     if (fused_pool_input) ss << ", AvePool 2x2 of " << fused_pool_input->h << "x" << fused_pool_input->w << " inside";
+    if (fused_maxpool_out) ss << " + MaxPool 3x3 stride 2" << (fused_maxpool_sign ? " + Sign" : "");
     return ss.str();
 }
 

@@ -121,7 +121,12 @@ void Net::add_mat(const std::string &name, std::shared_ptr<Mat> mat) { mat_map_[
 
 std::shared_ptr<Mat> Net::get_blob(const std::string &name) {
     auto it = mat_map_.find(name);
-    if (it == mat_map_.end()) throw std::out_of_range("Key " + name + " not found.");  // StrKeyMap::at, common/StrKeyMap.h
+    if (it == mat_map_.end()) {
+        auto gone = elided_.find(name);
+        if (gone != elided_.end())
+            throw std::runtime_error("blob " + name + " is not produced: " + gone->second + "; read the model with optimize = false to get it");
+        throw std::out_of_range("Key " + name + " not found.");  // StrKeyMap::at, common/StrKeyMap.h
+    }
     return it->second;
 }
 
@@ -311,7 +316,8 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
         writes = {bc->output_mat.get(), bc->binarized_mat.get(), bc->col_mat.get()};
     } else if (auto fc = std::dynamic_pointer_cast<FloatConv>(l)) {
         reads = {fc->fused_pool_input ? fc->fused_pool_input.get() : fc->input_mat.get()};
-        writes = {fc->output_mat.get()};
+        writes = {fc->output_mat ? fc->output_mat.get() : fc->fused_maxpool_out.get()};
+        if (fc->fused_maxpool_sign) writes.push_back(fc->fused_maxpool_sign.get());
         if (fc->fused_pool_input) writes.push_back(fc->input_mat.get());  // the pooled blob, a side product
     } else if (auto af = std::dynamic_pointer_cast<Affine>(l)) {
         reads = writes = {af->data_mat.get()};
@@ -351,6 +357,9 @@ static bool contains(const std::vector<const Mat *> &v, const Mat *m) {
 //     layer's packed input and the later layer skips its pack_mat.
 //  4. AvePool 2x2 stride 2 -> 1x1 FloatConv (the shortcut branch of a down-sampling block) becomes one launch that
 //     still writes the pooled blob.
+//  5. FloatConv (-> Affine -> Relu) -> MaxPool 3x3 stride 2 pad 1, the pool being the only reader of the convolution's
+//     blob (the stem), becomes one pass that never writes that blob when the library says the pass pays for these
+//     shapes; the blob leaves the net (get_blob says why) and its memory, four times the pooled blob's, is freed.
 void Net::fuse_binconv_epilogues() {
     std::vector<const Mat *> rd, wr;
     for (size_t i = 0; i + 2 < layers.size(); ++i) {
@@ -476,6 +485,40 @@ void Net::fuse_binconv_epilogues() {
         fc->fused_pool_input = pool->input_mat;
         layers.erase(layers.begin() + i);
         --i;
+    }
+
+    for (size_t i = 0; i + 1 < layers.size(); ++i) {
+        auto fc = std::dynamic_pointer_cast<FloatConv>(layers[i]);
+        auto pool = std::dynamic_pointer_cast<MaxPool>(layers[i + 1]);
+        if (!fc || !pool || fc->fused_pool_input || pool->input_mat != fc->output_mat || pool->kernel_h != 3 ||
+            pool->kernel_w != 3 || pool->stride_h != 2 || pool->stride_w != 2 || pool->pad_h != 1 || pool->pad_w != 1)
+            continue;
+        bool only_reader = true;
+        for (size_t j = 0; j < layers.size() && only_reader; ++j) {
+            if (j == i || j == i + 1) continue;
+            layer_io(layers[j], rd, wr);
+            if (contains(rd, fc->output_mat.get()) || contains(wr, fc->output_mat.get())) only_reader = false;
+        }
+        const Mat &in = *fc->input_mat;
+        const Mat &wt = *fc->weight_mat;
+        if (!only_reader || !dab_fconv_maxpool_pays(in.n, in.h, in.w, in.c, wt.h, wt.w, fc->pad_h, fc->pad_w, fc->stride_h,
+                                                    fc->stride_w, fc->dilation, fc->dilation, wt.n))
+            continue;
+        const int64_t carry = dab_fconv_maxpool_carry_floats(in.n, in.h, in.w, in.c, wt.h, wt.w, fc->pad_h, fc->pad_w,
+                                                             fc->stride_h, fc->stride_w, fc->dilation, fc->dilation, wt.n);
+        fc->fused_maxpool_out = pool->output_mat;
+        fc->fused_maxpool_sign = pool->fused_sign_out;
+        fc->fused_maxpool_carry = std::make_shared<Mat>((size_t)carry, DataType::Float, fc->name_ + "_carry");
+        for (auto it = mat_map_.begin(); it != mat_map_.end();) {
+            if (it->second == fc->output_mat) {
+                elided_[it->first] = "the convolution and the MaxPool behind it run as one pass";
+                it = mat_map_.erase(it);
+            } else {
+                ++it;
+            }
+        }
+        fc->output_mat.reset();
+        layers.erase(layers.begin() + i + 1);
     }
 }
 

@@ -55,6 +55,8 @@ class Net : public std::enable_shared_from_this<Net> {
     void *stream() const { return stream_; }
     void add_mat(const std::string &name, std::shared_ptr<Mat> mat);
     std::map<std::string, std::shared_ptr<Mat>> mat_map_;
+    // blobs of the model that the optimized layer list never writes (name -> why); get_blob names the reason
+    std::map<std::string, std::string> elided_;
 
    private:
     Net();

@@ -78,7 +78,7 @@ def run_model(layers, initializers, x, record=None):
 _INPLACE = {"Affine": "input", "Add": "input1", "Relu": "input", "PRelu": "input"}
 
 
-def run_segments(layers, initializers, fetch):
+def run_segments(layers, initializers, fetch, absent=()):
     """Layer-by-layer check with the other implementation's own activations as inputs.
 
     A sign network amplifies a one-ulp difference in a float layer into flipped bits downstream, so two correct
@@ -87,6 +87,8 @@ def run_segments(layers, initializers, fetch):
     final content of the input blobs as the implementation under test holds them after its run -- and yields
     (output blob name, type of the first layer, CPU result).  Valid when a blob is only read after the in-place layers
     on it have run, which holds for the graphs the converter emits (tools/onnx2bnn/OnnxConverter.cpp:583-639).
+    ``absent`` names blobs the implementation under test does not hold (it ran their producer and their one reader as
+    one pass): the reader's segment then continues the producer's instead of starting from a fetched blob.
     """
     blobs = {t["name"]: t for t in initializers}
     root = {}
@@ -101,6 +103,9 @@ def run_segments(layers, initializers, fetch):
         key = _INPLACE.get(layer["type"])
         if key is not None and r(layer[key]) in owner:
             owner[r(layer[key])].append(layer)  # joins the segment of the blob it rewrites, wherever that started
+        elif key is None and "input" in layer and r(layer["input"]) in absent and r(layer["input"]) in owner:
+            owner[r(layer["input"])].append(layer)  # reads a blob that only exists inside the other implementation's pass
+            owner[layer["output"]] = owner[r(layer["input"])]
         else:
             segs.append([layer])
             owner[r(layer[key]) if key is not None else layer["output"]] = segs[-1]

@@ -26,12 +26,24 @@ def close(got, want):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
 
 
-def check_every_segment(n, layers, inits, image):
+def blobs_not_produced(n, layers):
+    """Output names of the model whose blob the optimized layer list does not write (get_blob says so)."""
+    gone = set()
+    for layer in layers:
+        try:
+            n.blob_info(layer["output"])
+        except RuntimeError as e:
+            assert "is not produced" in str(e), str(e)
+            gone.add(layer["output"])
+    return gone
+
+
+def check_every_segment(n, layers, inits, image, absent=()):
     """Every layer group of the device run against the CPU restatement fed with the device's own input blobs:
     bit-exact after a binary convolution (counts are integers; Affine and Add round alike on both sides) and for
     max pooling, 1e-4 relative after float convolutions and average pooling."""
     checked = 0
-    for name, first_type, want in orc_net.run_segments(layers, inits, lambda b: n.get_blob(b)[image]):
+    for name, first_type, want in orc_net.run_segments(layers, inits, lambda b: n.get_blob(b)[image], absent):
         got = n.get_blob(name)[image]
         if first_type in ("BinConv2D", "MaxPool", "Affine", "Add", "Relu", "PRelu", "Concat"):
             np.testing.assert_array_equal(got, want, err_msg=name)
@@ -181,6 +193,40 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     descs = big.layers()
     assert sum("+ Sign" in d for d in descs) == 13 and sum("packed input from its producer" in d for d in descs) == 14
     big.close()
+
+
+@pytest.mark.parametrize("stem", [False, True])
+def test_bireal18_stem_and_maxpool_in_one_pass_at_batch_40(mods, stem):
+    """From a few dozen images on the last float convolution of the stem and the MaxPool behind it run as one pass that
+    never writes the convolution's blob: the pooled blob and the packed copy still match the CPU layers fed with the
+    device's own input, the elided blob is reported as such, and optimize = false brings it back."""
+    df, models, net = mods
+    layers, inits, inputs = models.bireal18(12, stem=stem)
+    buf = df.write_model(layers, inits, inputs)
+    batch = 40
+    x = np.random.default_rng(10).standard_normal((batch, 224, 224, 3)).astype(np.float32)
+    n = net.Net(batch=batch).read_buf(buf)
+    descs = n.layers()
+    assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == 1 and not any(d.startswith("MaxPool") for d in descs)
+    gone = blobs_not_produced(n, layers)
+    last_conv = "stem2_out" if stem else "conv1_out"
+    assert gone == {last_conv, last_conv + "_bn"} | ({last_conv + "_bn_relu"} if stem else set())
+    with pytest.raises(RuntimeError, match="is not produced: the convolution and the MaxPool"):
+        n.get_blob(last_conv)
+    n.run(x)
+    for i in (0, batch - 1):
+        assert check_every_segment(n, layers, inits, i, gone) >= 19
+        assert check_packed_inputs(n, layers, i) == 16
+    pooled = n.get_blob("pool1_out").copy()
+    n.close()
+    plain = net.Net(batch=batch, optimize=False).read_buf(buf)
+    assert blobs_not_produced(plain, layers) == set()
+    plain.run(x)
+    conv = plain.get_blob(last_conv)  # after the in-place Affine (and Relu)
+    for i in (0, 17, batch - 1):
+        want = orc.max_pool(conv[i], 3, 3, 1, 1, 2, 2)
+        close(pooled[i], want)
+    plain.close()
 
 
 def test_error_paths(mods, tmp_path):
