@@ -1,4 +1,5 @@
-"""Runs the float convolutions of the Bi-Real-18 stems at batch 256 a few times, for rocprofv3 runs.
+"""Runs the float convolutions of the Bi-Real-18 stems at batch 256 a few times, for rocprofv3 runs; the two that a
+MaxPool follows also as the one-pass kernel with the pool inside.
 
 usage: python3 -m dabnn_amd.profile_fconv    (prints the shapes it launched, in launch order)
 """
@@ -23,6 +24,13 @@ def main():
             dab.fconv_affine_relu(x, w, None, a, b, True, k, k, pad, pad, stride, stride)
         torch.cuda.synchronize()
         print("%dx%dx%dx%d -> %d, %dx%d stride %d" % (n, h, h, c, cout, k, k, stride))
+        if (h + 2 * pad - k) // stride + 1 == 112 and cout == 64:
+            # the last convolution of a stem with its MaxPool 3x3 stride 2 in one pass (no Relu in front of the pool
+            # of the 7x7 stem, one behind the 3x3 one -- the same instructions either way)
+            for _ in range(3):
+                dab.fconv_maxpool(x, w, None, a, b, True, k, k, pad, pad, stride, stride, want_sign=True)
+            torch.cuda.synchronize()
+            print("  the same + MaxPool 3x3 stride 2 + sign bits, one pass")
 
 
 if __name__ == "__main__":
