@@ -525,6 +525,13 @@ static bool plan_bands(int h, int w, int c, int kh, int kw, int pad_h, int pad_w
     return true;
 }
 
+// The shapes of the kernel that reads its operands from the raw input rows.
+static bool takes_raw_tile(int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h, int dil_w,
+                           const BandPlan &b) {
+    return c == 3 && kh == 7 && kw == 7 && stride_h == 2 && stride_w == 2 && pad_h == 3 && pad_w == 3 && dil_h == 1 &&
+           dil_w == 1 && b.ow == 112;
+}
+
 }  // namespace dab
 
 extern "C" int64_t dab_fconv_maxpool_carry_floats(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
@@ -538,10 +545,13 @@ extern "C" int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw
                                       int stride_w, int dil_h, int dil_w, int cout) {
     dab::BandPlan b;
     if (n <= 0 || !dab::plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b)) return 0;
-    // a band is a long work item and a CU holds one block: below several rounds of blocks the last round's idle CUs
-    // cost more than the saved traffic
+    // A band is a long work item (17-30 us) and a CU holds one block.  The raw-tile stem kernel beats the two launches
+    // as soon as the bands fill a good part of one round (measured: equal at 112 bands, 32 against 46 us at 224); the
+    // im2col band kernel gains less per band and needs several rounds before the last round's idle CUs stop mattering.
     const long long blocks = (long long)n * b.bands * ((cout + dab::kBandChannels - 1) / dab::kBandChannels);
-    return blocks >= 4ll * (dab::simd_count() / 4) ? 1 : 0;
+    const long long cus = dab::simd_count() / 4;
+    if (dab::takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) return 5 * blocks >= 3 * cus ? 1 : 0;
+    return blocks >= 4 * cus ? 1 : 0;
 }
 
 extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
@@ -585,8 +595,7 @@ extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, con
     if (items >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
     const int cus = simd_count() / 4;
     const dim3 grid((unsigned)(items < cus ? items : cus));
-    if (c == 3 && kh == 7 && kw == 7 && stride_h == 2 && stride_w == 2 && pad_h == 3 && pad_w == 3 && dil_h == 1 &&
-        dil_w == 1 && b.ow == 112) {
+    if (takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) {
         if (pooled_packed)
             hipLaunchKernelGGL(fconv7x7s2_maxpool_kernel<true>, grid, dim3(kBandThreads), 0, s, a);
         else
