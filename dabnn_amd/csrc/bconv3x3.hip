@@ -336,7 +336,7 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
     static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW>, 64 * kWavesPerBlock);
-    const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock);
+    const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
     a.div_groups = FastDiv((uint32_t)a.n_groups);

@@ -608,6 +608,9 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
         // a three-channel image too small for 128-pixel tiles (the stem at batch 1): 64-pixel tiles keep the
         // one-load-per-tap loader and still give most CUs a block
         DAB_FCONV_LAUNCH(64, 64, 24, 1, 3);
+    } else if (big_tiles < simd_count() / 4 && vec4 && ((M + 63) / 64) * ((cout + 63) / 64) >= simd_count() / 8) {
+        // fewer big tiles than CUs, but enough 64 x 64 ones for half of them: a wave still multiplies a whole 32 x 32 tile
+        DAB_FCONV_LAUNCH(64, 64, 16, 1, 4);
     } else if (big_tiles < simd_count() / 4) {
         // fewer big tiles than CUs: 32 x 32 tiles, each slice's depth split over the block's waves
         if (vec4)
@@ -671,7 +674,9 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
 #define DAB_POOLED_LAUNCH(BM, BN, SK, KSPLIT)                                                                     \
     hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false, 4, true>),                                        \
                        dim3((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN)), dim3(256), 0, s, a)
-    if (big_tiles < simd_count() / 4)
+    if (big_tiles < simd_count() / 4 && ((M + 63) / 64) * ((cout + 63) / 64) >= simd_count() / 8)
+        DAB_POOLED_LAUNCH(64, 64, 16, 1);
+    else if (big_tiles < simd_count() / 4)
         DAB_POOLED_LAUNCH(32, 32, 64, 4);
     else if (bn == 32)
         DAB_POOLED_LAUNCH(128, 32, 16, 1);

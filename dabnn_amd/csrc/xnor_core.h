@@ -361,12 +361,12 @@ inline int resident_blocks_per_cu(Kernel kernel, int block_threads) {
     return blocks;
 }
 
-inline int pick_wave_count(int n_items, int blocks_per_cu, int waves_per_block) {
+inline int pick_wave_count(int n_items, int blocks_per_cu, int waves_per_block, int units_per_item = 1) {
     long long w = (long long)(simd_count() / 4) * blocks_per_cu * waves_per_block;
     // Fewer items than resident waves: one item per wave.  When that still fills more than half of the machine,
-    // two items per wave are faster, because a wave fetches its lane-resident operand once for both; smaller
-    // problems are latency-bound and keep one item per wave.
-    if (w >= n_items) w = 2ll * n_items > w ? (n_items + 1) / 2 : n_items;
+    // two items per wave are faster, because a wave fetches its lane-resident operand once for both (items that are
+    // two units or more already share it); smaller problems are latency-bound and keep one item per wave.
+    if (w >= n_items) w = (2ll * n_items > w && units_per_item < 2) ? (n_items + 1) / 2 : n_items;
     if (w < 1) w = 1;
     return (int)((w + waves_per_block - 1) / waves_per_block * waves_per_block);
 }

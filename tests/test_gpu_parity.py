@@ -325,6 +325,8 @@ RTOL = 1e-4
     # a handful of pixels through a 1x1 convolution: the matrix-vector kernel (ragged channel count, 1 to 8 pixels)
     (1, 1, 512, 1000, 1, 0, 1, 1, True), (8, 1, 64, 70, 1, 0, 1, 1, False), (2, 2, 256, 65, 1, 0, 1, 1, True),
     (5, 1, 1024, 64, 1, 0, 1, 1, False),
+    # too few 128-row tiles for the CUs but plenty of 64 x 64 ones: ragged in both directions, padded and not
+    (3, 40, 32, 96, 3, 1, 1, 1, True), (2, 61, 8, 130, 1, 0, 1, 1, False),
 ])
 def test_fconv(dab, n, h, c, cout, k, pad, stride, dil, bias):
     r = rng(40)
