@@ -296,6 +296,16 @@ def main():
         t_img = time.perf_counter() - t1
         workloads["config4_5_bireal18"]["cpu_port_1_core"] = {"images/s": round(1.0 / t_img, 3), "ms": round(t_img * 1e3, 1),
                                                               "note": "CPU restatement of the reference layer loop, 1 image"}
+        # the reference is single-threaded and not re-entrant: more cores means independent processes, one image
+        # stream each (at most 16, the host share of a one-GPU box)
+        import multiprocessing
+        procs = max(1, min(16, os.cpu_count() or 1))
+        with multiprocessing.get_context("spawn").Pool(procs) as pool:
+            start_at = time.time() + 8.0 + 0.25 * procs  # after every worker's import and warm-up image
+            done = pool.map(orc_net.time_images, [(layers, inits, 3, 100 + i, start_at) for i in range(procs)])
+        workloads["config4_5_bireal18"]["cpu_port_all_cores"] = {
+            "images/s": round(sum(reps / t for reps, t in done), 2), "processes": procs,
+            "note": "independent processes of the CPU layer loop, one image stream each, 3 images per process"}
         cpu = {"value": done_ops / t_cpu, "unit": "binop/s", "cores": 1, "kind": "port",
                "sample": "%d passes of the 7 stage shapes at batch 1 through the reference's x86 dispatch "
                          "(pack_mat + baseline_bconv for 64 channels, fused_binarize_im2col + bgemm_naive "

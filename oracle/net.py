@@ -121,3 +121,18 @@ def run_segments(layers, initializers, fetch, absent=()):
                 act[layer["input2"]] = np.array(fetch(r(layer["input2"])), dtype=np.float32, copy=True)
             _apply(layer, act, blobs)
         yield r(seg[-1]["output"]), first["type"], act[seg[-1]["output"]]
+
+
+def time_images(job):
+    """Worker of a process pool: runs ``reps`` images through run_model after one warm-up image, all workers starting
+    at the wall-clock time ``start_at``; returns (reps, seconds).  job = (layers, initializers, reps, seed, start_at)."""
+    import time
+    layers, initializers, reps, seed, start_at = job
+    x = np.random.default_rng(seed).standard_normal((224, 224, 3)).astype(np.float32)
+    run_model(layers, initializers, x)
+    while time.time() < start_at:
+        time.sleep(0.001)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run_model(layers, initializers, x)
+    return reps, time.perf_counter() - t0
