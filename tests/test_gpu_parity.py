@@ -400,7 +400,9 @@ def test_affine_add_bit_exact(dab):
 
 
 @pytest.mark.parametrize("n,h,w,c,cout,affine", [(1, 56, 56, 64, 128, True), (2, 9, 7, 8, 5, False), (3, 28, 28, 128, 256, True),
-                                                 (1, 14, 14, 256, 512, True), (40, 56, 56, 64, 128, True), (1, 2, 2, 4, 8, False)])
+                                                 (1, 14, 14, 256, 512, True), (40, 56, 56, 64, 128, True), (1, 2, 2, 4, 8, False),
+                                                 # enough pixels for the 128-row tiles: one column tile (32-deep slices) and two
+                                                 (48, 56, 56, 64, 128, True), (170, 28, 28, 128, 256, False)])
 def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine):
     """The shortcut branch of a down-sampling block in one launch: the pooled tensor is bit for bit what ave_pool
     writes (and what the CPU restatement computes), the convolution bit for bit what fconv_affine_relu makes of it."""
