@@ -808,7 +808,11 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
         case 16: launch(pool_vec4_kernel<MAX, SIGN, 16>); break;                 \
         default: launch(pool_vec4_kernel<MAX, SIGN, 32>); break;                 \
     }
-        if (want_sign) {
+        if (!is_max && taps > 32 && taps <= 49 && v.total <= 4096u) {
+            // a global 7x7 average at batch 1-8: a few waves whose whole life is waiting for their taps -- ask for
+            // all 49 at once
+            launch(pool_vec4_kernel<false, false, 49>);
+        } else if (want_sign) {
             DAB_POOL_LAUNCH(true, true)
         } else if (is_max) {
             DAB_POOL_LAUNCH(true, false)

@@ -520,7 +520,10 @@ def test_concat_bit_exact(dab, n, h, w, ca, cb):
 
 
 @pytest.mark.parametrize("n,h,w,c,k,pad,stride", [(1, 8, 8, 4, 2, 0, 2), (2, 7, 7, 512, 7, 0, 1), (1, 9, 6, 4, 3, 1, 2),
-                                                  (1, 112, 112, 64, 3, 1, 2), (2, 56, 56, 64, 2, 0, 2)])
+                                                  (1, 112, 112, 64, 3, 1, 2), (2, 56, 56, 64, 2, 0, 2),
+                                                  # windows of up to 49 taps cut by the border, few enough outputs for the
+                                                  # all-taps-in-flight kernel; a 6x6 window; many outputs of a 7x7 one
+                                                  (1, 9, 9, 64, 7, 3, 2), (3, 12, 12, 32, 6, 2, 3), (8, 28, 28, 128, 7, 3, 1)])
 def test_pools(dab, n, h, w, c, k, pad, stride):
     x = rng(42).standard_normal((n, h, w, c)).astype(np.float32)
     avg = dab.ave_pool(dev_f(x), k, k, pad, pad, stride, stride).cpu().numpy()
