@@ -89,6 +89,23 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     if (i0 >= i1) return;
     const int u0 = i0 * S, u1 = i1 * S;
 
+    if constexpr (CW == 8) {
+        // The filters of 512 input channels are 295 KB and more that every wave walks through with scalar loads.
+        // When other kernels have run in between they are in no L2 any more, and the first wave to need a row waits
+        // for memory in the middle of its unit.  So the launch first touches every 128-byte line of the filters once
+        // per XCD (blocks are dealt to the eight XCDs in turn: block b runs on XCD b % 8): wave j of an XCD asks for
+        // one dword of each of the lines 64*j .. 64*j+63, straight into an LDS scratch line that nobody reads, with
+        // no register and no wait involved.
+        __shared__ uint32_t prefetch_dump[kWavesPerBlock * 64];
+        const uint32_t n_lines = (uint32_t)(p.cout * 9 * CW * 8) >> 7;
+        const uint32_t first = (uint32_t)((blockIdx.x >> 3) * kWavesPerBlock + wib) * 64u;
+        if (first < n_lines) {
+            const uint32_t line = first + lane < n_lines ? first + lane : n_lines - 1;
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1))) *)(reinterpret_cast<const unsigned char *>(p.w) + (size_t)line * 128),
+                (void __attribute__((address_space(3))) *)(prefetch_dump + wib * 64), 4, 0, 0);
+        }
+    }
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
     int tile = (int)p.div_groups.div((uint32_t)u0);
     int cg = u0 - tile * p.n_groups;
