@@ -1,14 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the binary-convolution hot path on one MI355X.
 
-Headline workload (BASELINE.json config 3 at batch 64): one "step" is one pass
+Headline workload (the seven ResNet-18 stage shapes at batch 64): one "step" is one pass
 of the direct 3x3 binary convolution over the seven ResNet-18 stage shapes
 (56/64, 28/128, 14/256, 7/512 at stride 1 and the three stride-2 channel
 doubling layers), packed activations and weights already resident in HBM,
 fp32 mismatch counts written back.  value = binary ops per second,
 binops = 2*N*OH*OW*Cout*9*Cin.
 
-The same JSON line also carries, under "workloads", the other BASELINE
+The same JSON line also carries, under "workloads", the other benchmark
 configurations (single 56x56x64 layer at batch 1, standalone bitpack and bgemm,
 the whole BinConv layer from fp32 input), the VALU-popcount roofline of the
 dominant kernel and the CPU baseline (the oracle's restatement of the

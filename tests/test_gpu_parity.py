@@ -1,7 +1,7 @@
 """GPU parity: HIP kernels (through the C ABI) vs the CPU oracle, bit-exact.
 
 Same seeded inputs go to both sides.  Sizes are chosen so the oracle finishes
-in seconds; the full BASELINE shapes at batch 64 are checked through
+in seconds; the benchmark's full shapes at batch 64 are checked through
 size-independent properties in test_gpu_properties.py.
 """
 import numpy as np
@@ -110,7 +110,7 @@ def test_fused_binarize_im2col_size_limit(dab):
     (159, 253, 68),  # tests/bgemm_test.cpp:12-27
     (128, 784, 18), (256, 196, 36), (512, 49, 72),  # tests/bgemm_test.cpp:132-181
     (33, 17, 10), (8, 64, 1), (16, 1, 9), (5, 70, 3), (1, 1, 1), (64, 130, 8), (72, 65, 25),
-    (512, 3136, 72),  # BASELINE config 2
+    (512, 3136, 72),  # the benchmark's standalone bgemm
 ])
 def test_bgemm_matches_naive(dab, m, n, k):
     a = rng(10).integers(0, 2**64, size=(k, m), dtype=np.uint64)
@@ -173,7 +173,7 @@ def test_im2col_transpose_bgemm_equals_baseline_bconv(dab):
     (1, 64, 64, 128, 128, 1, 1),  # tests/bconv_test.cpp bconv_test_3x3_128
     (1, 32, 32, 256, 256, 1, 1), (1, 16, 16, 512, 256, 1, 1), (1, 16, 16, 512, 1024, 2, 1),
     (1, 56, 56, 64, 64, 1, 1), (1, 28, 28, 128, 128, 1, 1), (1, 14, 14, 256, 256, 1, 1), (1, 7, 7, 512, 512, 1, 1),
-    (1, 56, 56, 64, 128, 2, 1), (1, 28, 28, 128, 256, 2, 1), (1, 14, 14, 256, 512, 2, 1),  # BASELINE config 3, batch 1
+    (1, 56, 56, 64, 128, 2, 1), (1, 28, 28, 128, 256, 2, 1), (1, 14, 14, 256, 512, 2, 1),  # the seven ResNet-18 stage shapes of the benchmark, batch 1
     # more than 1024 work items of 64 pixels x 8 channels: the unit kernel (everything above runs the small-problem
     # kernel), every channel count at stride 1 and 2, ragged last tiles, no padding, and the two narrow builds
     (6, 56, 56, 64, 64, 1, 1), (9, 28, 28, 128, 128, 1, 1), (17, 14, 14, 256, 256, 1, 1), (25, 7, 7, 512, 512, 1, 1),
@@ -272,7 +272,7 @@ def test_bconv_3x3_unsupported_and_invalid(dab):
 
 # ---------------------------------------------------------------- BinConv layer
 @pytest.mark.parametrize("n,h,w,c,cout,k,pad,stride,method", [
-    (1, 56, 56, 64, 64, 3, 1, 1, 0),  # BASELINE config 1
+    (1, 56, 56, 64, 64, 3, 1, 1, 0),  # the benchmark's single layer
     (2, 8, 8, 64, 32, 3, 1, 2, 0), (2, 8, 8, 128, 64, 3, 1, 1, 0), (1, 7, 7, 512, 16, 3, 1, 1, 0),
     (1, 6, 10, 192, 8, 3, 1, 1, 1),  # 192 channels -> im2col + bgemm
     (2, 9, 9, 128, 16, 5, 2, 2, 1),  # 5x5
@@ -295,7 +295,7 @@ def test_binconv_layer_matches_reference_dispatch(dab, n, h, w, c, cout, k, pad,
 
 
 def test_binconv_config1_k_minus_2cnt(dab):
-    """BASELINE config 1: counts, then K - 2*cnt through the folded affine, vs a float convolution."""
+    """The benchmark's single 56x56x64 layer: counts, then K - 2*cnt through the folded affine, vs a float convolution."""
     r = rng(32)
     x = r.standard_normal((1, 56, 56, 64)).astype(np.float32)
     wf = r.standard_normal((64, 3, 3, 64)).astype(np.float32)

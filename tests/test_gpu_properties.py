@@ -1,4 +1,4 @@
-"""GPU: BASELINE shapes at full batch size, checked through properties that do
+"""GPU: the benchmark's shapes at full batch size, checked through properties that do
 not need the CPU oracle to chew through billions of bit operations:
 
 * an independent textbook computation on the GPU itself: for +-1 tensors the
