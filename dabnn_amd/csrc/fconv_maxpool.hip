@@ -99,7 +99,7 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
                         const float prod = fa * v;
                         v = prod + fb;
                     }
-                    if constexpr (decltype(has_relu)::value) v = v > 0.f ? v : 0.f;
+                    if constexpr (decltype(has_relu)::value) v = v < 0.f ? 0.f : v;  // std::max(v, 0.f): a NaN stays
                     stage[(wm * (TM * 16) + i * 16 + 4 * f_s + e) * kStageStride + col] = v;
                 }
         }

@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
             const float prod = fa * v;
             v = prod + fb;
         }
-        if constexpr (decltype(has_relu)::value) v = v > 0.f ? v : 0.f;
+        if constexpr (decltype(has_relu)::value) v = v < 0.f ? 0.f : v;  // std::max(v, 0.f): a NaN stays
         __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), o_rsrc, (int)off, 0, 0);
     };
     // accumulator element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l % 32
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(256) void fconv_gemv_kernel(const FconvArgs p) {
                     const float prod = p.aff_a[co] * v;
                     v = prod + p.aff_b[co];
                 }
-                if (p.relu) v = v > 0.f ? v : 0.f;
+                if (p.relu) v = v < 0.f ? 0.f : v;
                 p.out[(size_t)(m0 + r) * p.cout + co] = v;
             }
         }
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256) void add_kernel(float *__restrict__ a, const f
 
 __global__ __launch_bounds__(256) void relu_kernel(float *__restrict__ x, long long total) {
     const long long stride = (long long)gridDim.x * 256;
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = x[i] > 0.f ? x[i] : 0.f;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) x[i] = x[i] < 0.f ? 0.f : x[i];
 }
 
 // PRelu.cpp:6-30: negative values are scaled by one slope or by their channel's slope (slope_n = 1 or c).

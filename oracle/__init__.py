@@ -297,6 +297,14 @@ def add_inplace(a, b):
     return a
 
 
+def relu_inplace(x):
+    """dabnn/layers/Relu.cpp:22-26: *ptr = std::max(*ptr, 0.f), i.e. (x < 0) ? 0 : x -- a NaN and a negative zero stay
+    what they are (numpy.maximum would return +0 for -0 on some builds)."""
+    assert x.dtype == np.float32
+    np.copyto(x, np.float32(0), where=x < 0)
+    return x
+
+
 def prelu_inplace(x, slope):
     assert x.dtype == np.float32 and x.flags["C_CONTIGUOUS"]
     slope, sp = _f(slope)

@@ -47,7 +47,7 @@ def _apply(layer, act, blobs, record=None):
         act[layer["output"]] = buf
     elif ty == "Relu":
         buf = act[layer["input"]]
-        np.maximum(buf, 0, out=buf)
+        orc.relu_inplace(buf)
         act[layer["output"]] = buf
     elif ty == "PRelu":
         buf = act[layer["input"]]

@@ -480,6 +480,16 @@ def test_fconv_maxpool_one_pass(dab, n, h, w, c, k, pad, stride, dil, cout, bias
     sep = dab.fconv_affine_relu(dev_f(xi), dev_f(wi), dev_f(bi) if bias else None, dev_f(ai) if affine else None,
                                 dev_f(ci) if affine else None, relu, k, k, pad, pad, stride, stride, dil, dil)
     np.testing.assert_array_equal(pooled.cpu().numpy(), dab.max_pool(sep, 3, 3, 1, 1, 2, 2).cpu().numpy())
+    # a NaN and an infinity in the image: the windows they reach are NaN (or infinite) after the convolution, and the
+    # pool passes over NaN as max_pool_fallback's comparison does
+    xi[0, h // 2, w // 3, :] = np.nan
+    xi[-1, h // 3, w // 2, 0] = np.inf
+    with np.errstate(invalid="ignore"):
+        want = cpu(xi, wi, bi, ai, ci)
+    pooled, packed = gpu(xi, wi, bi, ai, ci)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want)
+    if sign:
+        np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
 
 
 def test_fconv_maxpool_rejects_other_shapes(dab):
@@ -492,6 +502,25 @@ def test_fconv_maxpool_rejects_other_shapes(dab):
     with pytest.raises(RuntimeError, match="sign bits"):
         dab.fconv_maxpool(torch.zeros((1, 64, 56, 3), device="cuda"), torch.zeros((32, 7, 7, 3), device="cuda"), None, None,
                           None, False, 7, 7, 3, 3, 2, 2, want_sign=True)
+
+
+def test_relu_bit_exact_including_nan_and_negative_zero(dab):
+    """std::max(x, 0.f) of the reference keeps a NaN and a negative zero; so do the stand-alone kernel and the fused
+    epilogue of the float convolution."""
+    x = special_floats((2, 9, 7, 64), 52)
+    want = orc.relu_inplace(x.copy())
+    got = dab.relu_inplace(dev_f(x)).cpu().numpy()
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    # a 1x1 convolution with the identity as weights leaves the values as they are; zeros elsewhere in a row do not
+    # disturb a NaN or an infinity of the same pixel here, because every row of the identity has one non-zero entry
+    # and 0 * finite = 0 -- so take finite inputs plus NaN only
+    y = rng(53).standard_normal((1, 4, 4, 8)).astype(np.float32)
+    y[0, 1, 2, :] = np.nan
+    y[0, 0, 0, 0] = -0.0
+    eye = np.eye(8, dtype=np.float32).reshape(8, 1, 1, 8)
+    fused = dab.fconv_affine_relu(dev_f(y), dev_f(eye), None, None, None, True, 1, 1, 0, 0, 1, 1).cpu().numpy()
+    np.testing.assert_array_equal(np.isnan(fused), np.isnan(y))
+    np.testing.assert_array_equal(fused[~np.isnan(y)], np.maximum(y[~np.isnan(y)], 0))
 
 
 @pytest.mark.parametrize("shape", [(2, 5, 7, 64), (1, 3, 3, 5), (3, 16, 16, 192), (1, 1, 1, 1)])

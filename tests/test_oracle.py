@@ -357,6 +357,17 @@ def test_affine_and_add():
     np.testing.assert_array_equal(orc.add_inplace(x.copy(), y), x + y)
 
 
+def test_relu_known_answers():
+    """dabnn/layers/Relu.cpp:22-26 is std::max(x, 0.f) = (x < 0) ? 0 : x: negatives and -inf become +0, while -0, NaN,
+    denormals and +inf pass through bit for bit."""
+    x = np.array([-1.0, -0.0, 0.0, 1.0, np.nan, -np.inf, np.inf, -1e-40, 1e-40], np.float32)
+    want = np.array([0.0, -0.0, 0.0, 1.0, np.nan, 0.0, np.inf, 0.0, 1e-40], np.float32)
+    got = orc.relu_inplace(x.copy())
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    y = rng(51).standard_normal((3, 5, 8)).astype(np.float32)
+    np.testing.assert_array_equal(orc.relu_inplace(y.copy()), torch.relu(torch.from_numpy(y)).numpy())
+
+
 def test_prelu_vs_torch_and_concat_vs_numpy():
     """dabnn/layers/PRelu.cpp:6-30 against torch.nn.functional.prelu (NCHW, so the slope indexes dim 1) for one slope
     and for one slope per channel; dabnn/layers/Concat.cpp:7-21 against numpy.concatenate on the channel axis."""
