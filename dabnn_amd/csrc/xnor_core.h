@@ -366,7 +366,13 @@ inline int pick_wave_count(int n_items, int blocks_per_cu, int waves_per_block, 
     // Fewer items than resident waves: one item per wave.  When that still fills more than half of the machine,
     // two items per wave are faster, because a wave fetches its lane-resident operand once for both (items that are
     // two units or more already share it); smaller problems are latency-bound and keep one item per wave.
-    if (w >= n_items) w = (2ll * n_items > w && units_per_item < 2) ? (n_items + 1) / 2 : n_items;
+    if (w >= n_items) {
+        w = (2ll * n_items > w && units_per_item < 2) ? (n_items + 1) / 2 : n_items;
+        // the same number of waves on every SIMD where that costs few waves: a few more than a multiple of the SIMD count give some
+        // SIMDs one wave, and its items, more than the others get (3136 waves of two items: the SIMDs with four waves
+        // hold the launch until their eight items are done, the others have six)
+        if (w > simd_count() && (w % simd_count()) * 8 < simd_count()) w -= w % simd_count();
+    }
     if (w < 1) w = 1;
     return (int)((w + waves_per_block - 1) / waves_per_block * waves_per_block);
 }
