@@ -202,6 +202,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             ++cg;
         }
     }
+    // the filter prefetch wrote into this block's LDS: it has long arrived, but no wave leaves before that is certain
+    if constexpr (CW == 8) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
