@@ -232,6 +232,35 @@ def test_bireal18_stem_and_maxpool_in_one_pass_at_batch_40(mods, stem):
     plain.close()
 
 
+def test_stem_fusion_leaves_other_graphs_alone(mods):
+    """The convolution + MaxPool pass needs the pool to be the only reader of the convolution's blob and a 3x3 stride-2
+    pad-1 window: a second reader, or another window, keeps both layers, and every blob stays readable."""
+    df, models, net = mods
+    r = np.random.default_rng(13)
+    w = (r.standard_normal((64, 7, 7, 3)) / 12).astype(np.float32)
+    inits = [{"name": "w", "shape": [64, 7, 7, 3], "data": w, "align_hwc_to_128": False}]
+    conv = {"type": "FpConv2D", "name": "conv", "input": "data", "weight": "w", "output": "conv_out", "pads": [3] * 4,
+            "strides": [2, 2], "dilations": [1, 1]}
+    pool = {"type": "MaxPool", "name": "pool", "input": "conv_out", "output": "pool_out", "kernel_shape": [3, 3],
+            "pads": [1] * 4, "strides": [2, 2]}
+    other = {"type": "AvePool", "name": "avg", "input": "conv_out", "output": "avg_out", "kernel_shape": [2, 2],
+             "pads": [0] * 4, "strides": [2, 2]}
+    pool2 = dict(pool, kernel_shape=[2, 2], pads=[0] * 4)
+    batch = 8
+    x = r.standard_normal((batch, 224, 224, 3)).astype(np.float32)
+    for layers, fused in (([conv, pool], True), ([conv, pool, other], False), ([conv, pool2], False)):
+        n = net.Net(batch=batch).read_buf(df.write_model(layers, inits, [("data", [1, 224, 224, 3])]))
+        descs = n.layers()
+        assert any("+ MaxPool 3x3 stride 2" in d for d in descs) == fused, descs
+        assert len(descs) == (len(layers) - 1 if fused else len(layers))
+        n.run(x)
+        gone = blobs_not_produced(n, layers)
+        assert gone == ({"conv_out"} if fused else set())
+        for i in (0, batch - 1):
+            assert check_every_segment(n, layers, inits, i, gone) == len(layers) - len(gone)
+        n.close()
+
+
 def test_error_paths(mods, tmp_path):
     df, models, net = mods
     with pytest.raises(ValueError, match="Open file error"):  # std::invalid_argument, dabnn/net.cpp:34-36
