@@ -335,7 +335,9 @@ __global__ __launch_bounds__(256) void bconv3x3_ksplit_kernel(const BconvArgs p)
 // So few work items (64 pixels x 8 channels) that splitting each over four waves gives a SIMD four waves at most
 // (measured on Bi-Real-18 at batch 1 to 16: faster than the unit kernel up to there).
 static bool splits_depth(long long tiles, int cin, int cout) {
-    return tiles * (cout / 8) <= simd_count();
+    // 512 input channels: a unit there is 72 scalar loads of filters per channel, and the kernel that keeps an item's
+    // filters in LDS stays ahead up to eight waves per SIMD (7x7 512->512 at batch 24 and 32: 4-6 % of the whole net)
+    return tiles * (cout / 8) <= (long long)simd_count() * (cin >= 512 ? 2 : 1);
 }
 
 template <int CW, int MODE>

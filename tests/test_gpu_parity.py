@@ -174,10 +174,10 @@ def test_im2col_transpose_bgemm_equals_baseline_bconv(dab):
     (1, 32, 32, 256, 256, 1, 1), (1, 16, 16, 512, 256, 1, 1), (1, 16, 16, 512, 1024, 2, 1),
     (1, 56, 56, 64, 64, 1, 1), (1, 28, 28, 128, 128, 1, 1), (1, 14, 14, 256, 256, 1, 1), (1, 7, 7, 512, 512, 1, 1),
     (1, 56, 56, 64, 128, 2, 1), (1, 28, 28, 128, 256, 2, 1), (1, 14, 14, 256, 512, 2, 1),  # the seven ResNet-18 stage shapes of the benchmark, batch 1
-    # more than 1024 work items of 64 pixels x 8 channels: the unit kernel (everything above runs the small-problem
+    # more than 1024 work items of 64 pixels x 8 channels (2048 with 512 input channels): the unit kernel (everything above runs the small-problem
     # kernel), every channel count at stride 1 and 2, ragged last tiles, no padding, and the two narrow builds
     (6, 56, 56, 64, 64, 1, 1), (9, 28, 28, 128, 128, 1, 1), (17, 14, 14, 256, 256, 1, 1), (25, 7, 7, 512, 512, 1, 1),
-    (10, 56, 56, 64, 128, 2, 1), (20, 28, 28, 128, 256, 2, 1), (30, 14, 14, 256, 512, 2, 1), (40, 9, 9, 64, 272, 1, 0),
+    (10, 56, 56, 64, 128, 2, 1), (20, 28, 28, 128, 256, 2, 1), (30, 14, 14, 256, 512, 2, 1), (40, 9, 9, 64, 272, 1, 0), (48, 7, 7, 512, 512, 1, 1),
     (64, 56, 56, 64, 64, 1, 1), (200, 28, 28, 128, 128, 1, 1),
 ])
 def test_bconv_3x3_matches_baseline_bconv(dab, n, h, w, cin, cout, stride, pad):
@@ -204,7 +204,7 @@ def test_bconv_3x3_equals_pad_then_bconv_on_padded(dab):
     (2, 9, 7, 64, 64, 1, True), (1, 14, 14, 256, 256, 1, True), (3, 8, 8, 128, 24, 2, True), (1, 7, 7, 512, 64, 1, False),
     (5, 13, 13, 64, 72, 1, True), (1, 56, 56, 64, 64, 1, True),
     # the unit kernel (more than 1024 work items)
-    (6, 56, 56, 64, 64, 1, True), (9, 28, 28, 128, 72, 1, True), (17, 14, 14, 256, 256, 1, False), (25, 7, 7, 512, 512, 1, True),
+    (6, 56, 56, 64, 64, 1, True), (9, 28, 28, 128, 72, 1, True), (17, 14, 14, 256, 256, 1, False), (25, 7, 7, 512, 512, 1, True), (48, 7, 7, 512, 512, 1, True),
     (20, 28, 28, 128, 256, 2, True),
 ])
 def test_bconv_affine_add_equals_three_reference_layers(dab, n, h, w, cin, cout, stride, with_shortcut):
@@ -230,7 +230,7 @@ def test_bconv_affine_add_equals_three_reference_layers(dab, n, h, w, cin, cout,
     (3, 28, 28, 128, 128, 1, True), (70, 5, 5, 256, 64, 1, False),
     # the unit kernel (more than 1024 work items)
     (6, 56, 56, 64, 64, 1, True), (9, 28, 28, 128, 128, 1, True), (17, 14, 14, 256, 256, 1, True), (25, 7, 7, 512, 512, 1, True),
-    (30, 14, 14, 256, 512, 2, False), (10, 56, 56, 64, 128, 2, True),
+    (30, 14, 14, 256, 512, 2, False), (10, 56, 56, 64, 128, 2, True), (48, 7, 7, 512, 512, 1, True),
 ])
 def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, stride, with_shortcut):
     """The fp32 result equals the three reference layers, and the packed copy is pack_mat of that result, bit for bit

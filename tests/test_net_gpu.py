@@ -189,12 +189,12 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     assert "Bin Conv" in report and "Float Conv" in report and "total" in report
     n.close()
     # at a larger batch the two producers with 512 input channels leave the packing to their successors
-    big = net.Net(batch=32).read(str(path))
+    big = net.Net(batch=48).read(str(path))
     descs = big.layers()
     assert sum("+ Sign" in d for d in descs if d.startswith("Bin Conv")) == 13
     assert sum("packed input from its producer" in d for d in descs) == 14
-    # and the 7x7 stem runs with its MaxPool inside (from a handful of images on)
-    assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == (0 if stem else 1)
+    # and the last convolution of either stem runs with its MaxPool inside
+    assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == 1
     big.close()
 
 
