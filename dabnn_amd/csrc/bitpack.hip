@@ -6,7 +6,9 @@
 // A wave therefore reads 64 consecutive floats per instruction (256 coalesced
 // bytes), keeps the 64 masks of a 16 KiB chunk in lane i of a register pair
 // and writes them with one coalesced 512-byte store.  HBM-bound: 4 bytes read
-// and 1/16 byte written per element.
+// and 1/16 byte written per element.  Every float is read once, so the loads
+// are non-temporal (411 MB: 69 instead of 78 us); the words are stored the
+// ordinary way, the next kernel reads them.
 #include "common.h"
 
 namespace dab {
@@ -27,7 +29,7 @@ __global__ __launch_bounds__(64 * kPackWavesPerBlock) void bitpack_nhwc_kernel(c
         if (w0 + 64 <= n_words) {
 #pragma unroll 16
             for (int i = 0; i < 64; ++i) {
-                const uint64_t word = __ballot(src[(long long)i * 64] > 0.0f);
+                const uint64_t word = __ballot(__builtin_nontemporal_load(src + (long long)i * 64) > 0.0f);
                 mine = (lane == i) ? word : mine;
             }
             out[w0 + lane] = mine;
@@ -56,9 +58,9 @@ __global__ __launch_bounds__(256) void bitpack_nchw_kernel(const float *__restri
     const float *src = x + ((img * cw + k) * 64) * hw + pix;
     uint32_t lo = 0, hi = 0;
 #pragma unroll 8
-    for (int j = 0; j < 32; ++j) lo |= (src[(long long)j * hw] > 0.0f ? 1u : 0u) << j;
+    for (int j = 0; j < 32; ++j) lo |= (__builtin_nontemporal_load(src + (long long)j * hw) > 0.0f ? 1u : 0u) << j;
 #pragma unroll 8
-    for (int j = 0; j < 32; ++j) hi |= (src[(long long)(j + 32) * hw] > 0.0f ? 1u : 0u) << j;
+    for (int j = 0; j < 32; ++j) hi |= (__builtin_nontemporal_load(src + (long long)(j + 32) * hw) > 0.0f ? 1u : 0u) << j;
     out[(img * hw + pix) * cw + k] = ((uint64_t)hi << 32) | lo;
 }
 
