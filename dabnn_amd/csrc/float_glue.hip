@@ -688,7 +688,10 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
         // 256 x 56 x 56 x 64 -> 128)
         DAB_POOLED_LAUNCH(128, 128, 32, 1);
     else
-        DAB_POOLED_LAUNCH(128, 128, 16, 1);
+        // several column tiles: every one of them pools the input again, so the tile is as wide as the accumulators
+        // allow and 64 rows high (256 x 28 x 28 x 128 -> 256: 60 -> 55 us, 256 x 14 x 14 x 256 -> 512: 59 -> 48 us;
+        // 128 x 64 tiles: 90 us)
+        DAB_POOLED_LAUNCH(64, 256, 16, 1);
 #undef DAB_POOLED_LAUNCH
     DAB_LAUNCH_CHECK();
     return DAB_OK;

@@ -401,8 +401,11 @@ def test_affine_add_bit_exact(dab):
 
 @pytest.mark.parametrize("n,h,w,c,cout,affine", [(1, 56, 56, 64, 128, True), (2, 9, 7, 8, 5, False), (3, 28, 28, 128, 256, True),
                                                  (1, 14, 14, 256, 512, True), (40, 56, 56, 64, 128, True), (1, 2, 2, 4, 8, False),
-                                                 # enough pixels for the 128-row tiles: one column tile (32-deep slices) and two
-                                                 (48, 56, 56, 64, 128, True), (170, 28, 28, 128, 256, False)])
+                                                 # enough pixels for the large tiles: one column tile (128 rows, 32-deep
+                                                 # slices), more than 128 output channels (64 rows x 256 columns), the
+                                                 # latter with a ragged last tile both ways
+                                                 (48, 56, 56, 64, 128, True), (170, 28, 28, 128, 256, False),
+                                                 (97, 30, 30, 64, 200, True), (256, 14, 14, 256, 512, True)])
 def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine):
     """The shortcut branch of a down-sampling block in one launch: the pooled tensor is bit for bit what ave_pool
     writes (and what the CPU restatement computes), the convolution bit for bit what fconv_affine_relu makes of it."""
