@@ -162,3 +162,28 @@ def test_fconv_full_size_against_torch(dab, n, hw, c, cout, k, pad, stride):
     fused = dab.fconv_affine_relu(x, w, bias, a, b, True, k, k, pad, pad, stride, stride)
     ref2 = torch.relu(ref * a + b)
     assert (fused - ref2).abs().max().item() <= 1e-4 * max(ref2.abs().max().item(), scale * a.abs().max().item())
+
+
+@pytest.mark.parametrize("n,hw,c,cout,k,pad,stride,relu", [(256, 224, 3, 64, 7, 3, 2, False), (64, 112, 32, 64, 3, 1, 1, True),
+                                                            (7, 224, 3, 64, 7, 3, 2, True)])
+def test_fconv_maxpool_full_size_against_torch(dab, n, hw, c, cout, k, pad, stride, relu):
+    """The last convolution of either Bi-Real-18 stem with its MaxPool 3x3 stride 2 inside, at the real sizes (every
+    persistent block walks many bands), against torch's fp32 convolution and max pooling on the GPU, 1e-4 relative;
+    the packed copy is pack_mat of the pooled tensor the launch wrote."""
+    gen = torch.Generator().manual_seed(n + hw + c)
+    x = torch.randn((n, hw, hw, c), generator=gen).cuda()
+    w = (torch.randn((cout, k, k, c), generator=gen) / (k * k * c) ** 0.5).cuda()
+    a, b = torch.randn(cout, generator=gen).cuda(), torch.randn(cout, generator=gen).cuda()
+    torch.backends.cudnn.allow_tf32 = False
+    torch.backends.cuda.matmul.allow_tf32 = False
+    assert dab.fconv_maxpool_pays(n, hw, hw, c, k, k, pad, pad, stride, stride, 1, 1, cout)
+    ref = F.conv2d(x.permute(0, 3, 1, 2), w.permute(0, 3, 1, 2), None, stride=stride, padding=pad)
+    ref = ref * a.view(1, -1, 1, 1) + b.view(1, -1, 1, 1)
+    scale = ref.abs().max().item()
+    if relu:
+        ref = torch.relu(ref)
+    ref = F.max_pool2d(ref, 3, 2, 1).permute(0, 2, 3, 1)
+    pooled, packed = dab.fconv_maxpool(x, w, None, a, b, relu, k, k, pad, pad, stride, stride, want_sign=True)
+    assert pooled.shape == ref.shape
+    assert (pooled - ref).abs().max().item() <= 1e-4 * scale
+    assert torch.equal(packed, dab.pack_mat(pooled))
