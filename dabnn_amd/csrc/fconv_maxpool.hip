@@ -37,8 +37,23 @@ struct FconvPoolArgs {
     int band_rows, bands;  // R, bands per image
     int ph, pw;
     int ytiles;  // 64-channel tiles of cout
+    // chained: block b takes the items [b*per + min(b, extra), ...) one after the other (ytiles == 1: consecutive
+    // bands of an image) and keeps a band's last row for the next one in registers; otherwise the items gridDim.x apart
+    int chained, per, extra;
     FastDiv div_ow, div_c, div_kw, div_bands, div_ytiles;
 };
+
+// The work items of a block: first, one past the last, and the distance between two of them.
+struct BandRange {
+    int first, end, step;
+};
+__device__ __forceinline__ BandRange band_range(const FconvPoolArgs &p) {
+    const int b = (int)blockIdx.x;
+    if (!p.chained) return BandRange{b, p.n * p.bands * p.ytiles, (int)gridDim.x};
+    const int first = b * p.per + (b < p.extra ? b : p.extra);
+    return BandRange{first, first + p.per + (b < p.extra ? 1 : 0), 1};
+}
+constexpr int kKeepSlots = 4;  // pooled columns x 16 channel groups per thread: at most 112 * 16 / 512
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
@@ -74,9 +89,10 @@ struct BandOut {
 // A finished band (a wave's accumulators: 7 x 2 tiles of 16 pixels x 16 channels, wave (wm, wn) = pixels 112*wm ..,
 // channels 32*wn ..) goes through LDS to the pooled tensor, the carry and the sign bits.  All threads of the block
 // call it after a barrier that ended every other use of `stage`.
-template <bool SIGN>
+template <bool SIGN, int SLOTS>
 __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *stage, const f32x4v (&acc)[7][2], const BandOut o,
-                                              int tid, int wm, int wn, int f_s, int f_i) {
+                                              int tid, int wm, int wn, int f_s, int f_i, float4 (&keep)[SLOTS],
+                                              bool fold, bool write_carry) {
     constexpr int TM = 7, TN = 2;
     // The band goes to LDS (the slices are dead: the loop ended with a barrier): + bias, Affine (a*v + b, two
     // roundings), Relu, in the reference's order.  Accumulator element e of lane l: pixel 4*(l/16) + e, channel l % 16.
@@ -121,14 +137,19 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
     // Pooling: a thread takes four channels of one pooled column and walks down the band's rows.  h = the maximum
     // of the row's three columns 2*px-1 .. 2*px+1 (the first pooled column has two; one is read twice).  Pooled
     // row q is max(h[2q-1], h[2q], h[2q+1]); for q = 0 the row above the band is left out: row -1 of the image
-    // does not exist, and the last row of the band above arrives through the carry, which is this band's h[R-1].
-    for (int it = tid; it < p.pw * 16; it += kBandThreads) {
+    // does not exist, and the last row of the band above arrives through the carry, which is this band's h[R-1] --
+    // or, when this block made the band above just before (fold), it is in `keep`: a thread has the same columns
+    // and channels in every band.
+#pragma unroll
+    for (int slot = 0; slot < SLOTS; ++slot) {
+        const int it = tid + slot * kBandThreads;
+        if (it >= p.pw * 16) break;
         const int c4 = it & 15, px = it >> 4;
         const int co = o.n0 + c4 * 4;
         const float *col0 = &stage[(px == 0 ? 0 : 2 * px - 1) * kStageStride + c4 * 4];
         const float *col1 = &stage[(2 * px) * kStageStride + c4 * 4];
         const float4 lowest = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
-        float4 prev = lowest, even = lowest;
+        float4 prev = fold ? keep[slot] : lowest, even = lowest;
         for (int r = 0; r < p.band_rows; ++r) {
             const int ro = r * p.ow * kStageStride;
             const float4 h = max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
@@ -150,11 +171,12 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
                     }
                 }
             } else {
-                even = max3(prev, h, lowest);  // r == 0: prev is the lowest value, the row above is left out
+                even = max3(prev, h, lowest);  // r == 0 without fold: prev is the lowest value, the row above is left out
             }
             prev = h;
         }
-        if (co < p.cout) {
+        keep[slot] = prev;
+        if (write_carry && co < p.cout) {
             const float4 m = max3(prev, lowest, lowest);
             *reinterpret_cast<float4 *>(p.carry + ((size_t)(o.img * p.bands + o.band) * p.pw + px) * p.cout + co) = m;
         }
@@ -251,9 +273,13 @@ __global__ __launch_bounds__(kBandThreads) void fconv_maxpool_kernel(const Fconv
     // four slots does not matter as long as both operands agree: a lane reads two consecutive depths at once and
     // uses them in two instructions.
     const int f_s = lane >> 4, f_i = lane & 15;
-    const int n_items = p.n * p.bands * p.ytiles;
-    int item = blockIdx.x;
-    if (item >= n_items) return;
+    const BandRange range = band_range(p);
+    int item = range.first;
+    if (item >= range.end) return;
+    float4 keep[kKeepSlots];
+#pragma unroll
+    for (int slot = 0; slot < kKeepSlots; ++slot) keep[slot] = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+    bool fold = false;
     enter(item);
     fetch(0);
     for (;;) {
@@ -295,15 +321,19 @@ __global__ __launch_bounds__(kBandThreads) void fconv_maxpool_kernel(const Fconv
         // what the epilogue needs of this band, then the next band's first slice is asked for: its latency hides
         // behind the epilogue
         const int e_img = img, e_band = band, e_row0 = row0, e_n0 = n0;
-        const int next = item + gridDim.x;
-        const bool has_next = next < n_items;
+        const int next = item + range.step;
+        const bool has_next = next < range.end;
         if (has_next) {
             enter(next);
             fetch(0);
         }
 
-        band_epilogue<SIGN>(p, smem, acc, BandOut{e_img, e_band, e_row0, e_n0, e_n0 / BN}, tid, wm, wn, f_s, f_i);
+        // chained: the band above was this block's previous item unless this is its first one or an image's first
+        // band; the carry goes to memory only where another block continues
+        band_epilogue<SIGN, kKeepSlots>(p, smem, acc, BandOut{e_img, e_band, e_row0, e_n0, e_n0 / BN}, tid, wm, wn, f_s, f_i, keep,
+                            fold && e_band > 0, !p.chained || !has_next);
         if (!has_next) break;
+        fold = p.chained != 0;
         item = next;
         __syncthreads();  // the staged band is dead
     }
@@ -324,6 +354,8 @@ constexpr int kFilterStride = 148;                  // 7 x (16 + 4) + 7 + 1 floa
 constexpr int kFilterFloats = kBandChannels * kFilterStride;
 constexpr int kStemLdsFloats = kFilterFloats + kBandPixels * kStageStride;  // the tile shares the staged band's space
 constexpr int kTileLoads = (kTileRows * kTilePixels + kBandThreads - 1) / kBandThreads;
+constexpr int kStemKeepSlots = 2;  // 56 pooled columns x 16 channel groups on 512 threads
+static_assert(56 * 16 <= kStemKeepSlots * kBandThreads, "pooled columns of the stem");
 
 template <bool SIGN>
 __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const FconvPoolArgs p) {
@@ -336,9 +368,13 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
     const int wm = wave >> 1, wn = wave & 1;
     const int f_s = lane >> 4, f_i = lane & 15;
     const uint32_t img_bytes = (uint32_t)(p.h * p.wd * 3) * 4u;
-    const int n_items = p.n * p.bands * p.ytiles;
-    int item = blockIdx.x;
-    if (item >= n_items) return;
+    const BandRange range = band_range(p);
+    int item = range.first;
+    if (item >= range.end) return;
+    float4 keep[kStemKeepSlots];
+#pragma unroll
+    for (int slot = 0; slot < kStemKeepSlots; ++slot) keep[slot] = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+    bool fold = false;
 
     // the thread's pixels of a tile: byte offset from the tile's first row in the image, and place in LDS
     uint32_t t_off[kTileLoads];
@@ -403,8 +439,8 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         __syncthreads();
 
         const BandOut o{img, band, row0, n0, n0 / BN};
-        const int next = item + gridDim.x;
-        const bool has_next = next < n_items;
+        const int next = item + range.step;
+        const bool has_next = next < range.end;
         if (has_next) {
             enter(next);
             fetch_tile();
@@ -458,8 +494,9 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
                 }
         }
         __syncthreads();  // the tile is dead: the staged band takes its place
-        band_epilogue<SIGN>(p, tile, acc, o, tid, wm, wn, f_s, f_i);
+        band_epilogue<SIGN, kStemKeepSlots>(p, tile, acc, o, tid, wm, wn, f_s, f_i, keep, fold && o.band > 0, !p.chained || !has_next);
         if (!has_next) break;
+        fold = p.chained != 0;
         item = next;
         __syncthreads();  // the staged band is dead
     }
@@ -469,9 +506,10 @@ struct CarryArgs {
     float4 *pooled;
     const float4 *carry;
     uint64_t *bits;
-    uint32_t total;  // n * (bands - 1) * pw * c4
+    uint32_t total;  // n * (bands - 1) * pw * c4, chained: (blocks of the band kernel - 1) * pw * c4
     int bands, ph, pw, c4, half;
-    FastDiv div_c4, div_pw, div_bm1;
+    int chained, per, extra;  // as in FconvPoolArgs: only the first band of a block's range is left to do
+    FastDiv div_c4, div_pw, div_bm1, div_bands;
 };
 
 // pooled[first row of band b] = max(itself, carry of band b - 1), b >= 1; SIGN: and that row's sign bits again.
@@ -483,8 +521,18 @@ __global__ __launch_bounds__(256) void maxpool_carry_kernel(const CarryArgs p) {
     const int ch = (int)(idx - t * p.c4);
     uint32_t t2 = p.div_pw.div(t);
     const int px = (int)(t - t2 * p.pw);
-    const uint32_t img = p.div_bm1.div(t2);
-    const int b = (int)(t2 - img * (p.bands - 1)) + 1;
+    uint32_t img;
+    int b;
+    if (p.chained) {
+        const int blk = (int)t2 + 1;  // block 0 starts with an image's first band
+        const uint32_t item = (uint32_t)(blk * p.per + (blk < p.extra ? blk : p.extra));
+        img = p.div_bands.div(item);
+        b = (int)(item - img * p.bands);
+        if (b == 0) return;  // the 16 lanes of a pixel's word leave together
+    } else {
+        img = p.div_bm1.div(t2);
+        b = (int)(t2 - img * (p.bands - 1)) + 1;
+    }
     const size_t pix = ((size_t)img * p.ph + (size_t)b * p.half) * p.pw + px;
     const float4 m = p.pooled[pix * p.c4 + ch];
     const float4 v = p.carry[(((size_t)img * p.bands + (b - 1)) * p.pw + px) * p.c4 + ch];
@@ -519,6 +567,7 @@ static bool plan_bands(int h, int w, int c, int kh, int kw, int pad_h, int pad_w
     if (b.band_rows % 2 != 0 || b.ow % 2 != 0 || b.oh % b.band_rows != 0) return false;
     b.bands = b.oh / b.band_rows;
     b.ph = b.oh / 2, b.pw = b.ow / 2;  // out_dim(oh, 1, 3, 1, 2) for even oh
+    if (b.pw * 16 > kKeepSlots * kBandThreads) return false;  // (ow <= 224 here: never)
     if (cout % 4 != 0 || !(c == 3 || c % 4 == 0)) return false;
     // one image, 64 filters and 64 output pixels' worth of offsets stay below 2^30 bytes
     if (((long long)h + (long long)kh * dil_h + pad_h) * w * c * 4 >= (1ll << 30) || 64ll * kh * kw * c * 4 >= (1ll << 30)) return false;
@@ -595,6 +644,8 @@ extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, con
     if (items >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
     const int cus = simd_count() / 4;
     const dim3 grid((unsigned)(items < cus ? items : cus));
+    a.chained = a.ytiles == 1 && b.bands > 1;
+    a.per = (int)(items / grid.x), a.extra = (int)(items % grid.x);
     if (takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) {
         if (pooled_packed)
             hipLaunchKernelGGL(fconv7x7s2_maxpool_kernel<true>, grid, dim3(kBandThreads), 0, s, a);
@@ -617,12 +668,16 @@ extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, con
         ca.pooled = reinterpret_cast<float4 *>(pooled), ca.carry = reinterpret_cast<const float4 *>(carry);
         ca.bits = pooled_packed;
         ca.bands = b.bands, ca.ph = b.ph, ca.pw = b.pw, ca.c4 = cout / 4, ca.half = b.band_rows / 2;
-        const long long total = (long long)n * (b.bands - 1) * b.pw * ca.c4;
+        ca.chained = a.chained, ca.per = a.per, ca.extra = a.extra;
+        const long long total = (a.chained ? (long long)grid.x - 1 : (long long)n * (b.bands - 1)) * b.pw * ca.c4;
         if (total >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
         ca.total = (uint32_t)total;
         ca.div_c4 = FastDiv((uint32_t)ca.c4), ca.div_pw = FastDiv((uint32_t)b.pw), ca.div_bm1 = FastDiv((uint32_t)(b.bands - 1));
+        ca.div_bands = FastDiv((uint32_t)b.bands);
         const unsigned blocks = (unsigned)((total + 255) / 256);
-        if (pooled_packed)
+        if (total == 0) {
+            // one block made every band
+        } else if (pooled_packed)
             hipLaunchKernelGGL(maxpool_carry_kernel<true>, dim3(blocks), dim3(256), 0, s, ca);
         else
             hipLaunchKernelGGL(maxpool_carry_kernel<false>, dim3(blocks), dim3(256), 0, s, ca);

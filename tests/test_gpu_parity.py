@@ -437,6 +437,10 @@ def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine)
     # the 7x7 stride-2 stem at output width 112 has a kernel of its own: odd image sizes, two channel tiles on one
     # block, a ragged channel tile, a single band
     (2, 31, 223, 3, 7, 3, 2, 1, 128, True, True, True), (1, 8, 224, 3, 7, 3, 2, 1, 20, False, False, False),
+    # more bands than blocks: a block makes consecutive bands and hands the last row of one to the next in registers
+    # (ranges of one and two bands here, some across two images)
+    (12, 224, 224, 3, 7, 3, 2, 1, 64, False, True, False), (100, 32, 56, 4, 3, 1, 1, 1, 64, True, True, True),
+    (90, 16, 224, 4, 3, 1, 1, 1, 8, False, False, True),
 ])
 def test_fconv_maxpool_one_pass(dab, n, h, w, c, k, pad, stride, dil, cout, bias, affine, relu):
     """FpConv2D (+ Affine + Relu) + MaxPool 3x3 stride 2 pad 1 without the convolution's output in memory: within
