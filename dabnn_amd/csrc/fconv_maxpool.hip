@@ -594,13 +594,18 @@ extern "C" int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw
                                       int stride_w, int dil_h, int dil_w, int cout) {
     dab::BandPlan b;
     if (n <= 0 || !dab::plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b)) return 0;
-    // A band is a long work item (17-30 us) and a CU holds one block.  The raw-tile stem kernel beats the two launches
-    // as soon as the bands fill a good part of one round (measured: equal at 112 bands, 32 against 46 us at 224); the
-    // im2col band kernel gains less per band and needs several rounds before the last round's idle CUs stop mattering.
+    // A band is a long work item (17-45 us) and a CU holds one block, so a launch takes whole rounds of bands.  The
+    // raw-tile stem kernel beats the two launches from 140 bands on (measured at 84 to 812 bands: 31 against 33 us at
+    // 140, 33 against 46 at 224, 87 against 103 at 812; 2 us behind only at 280, just past a round; at 112 bands
+    // equal alone and 4 % behind inside Bi-Real-18, whose next layer then starts late).  The im2col band
+    // kernel gains a few per cent over full rounds and loses as much as the last round is empty (32 -> 64 channels at
+    // 112 x 112, one pass against two launches: 127 / 128 us at 672 bands, 166 / 143 at 784, 166 / 166 at 896,
+    // 205 / 187 at 1036): it runs when the last round leaves less than an eighth of all slots idle.
     const long long blocks = (long long)n * b.bands * ((cout + dab::kBandChannels - 1) / dab::kBandChannels);
     const long long cus = dab::simd_count() / 4;
-    if (dab::takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) return 5 * blocks >= 3 * cus ? 1 : 0;
-    return blocks >= 4 * cus ? 1 : 0;
+    if (dab::takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) return 2 * blocks > cus ? 1 : 0;
+    const long long rounds = (blocks + cus - 1) / cus;
+    return 8 * blocks > 7 * rounds * cus ? 1 : 0;
 }
 
 extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
