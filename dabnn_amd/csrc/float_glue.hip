@@ -477,7 +477,7 @@ struct PoolVecArgs {
 template <bool MAX, bool SIGN, int U>
 __global__ __launch_bounds__(256) void pool_vec4_kernel(const float4 *__restrict__ x, float4 *__restrict__ out,
                                                         uint64_t *__restrict__ out_packed, const PoolVecArgs p) {
-    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= p.total) return;
     uint32_t t = p.div_c4.div(idx);
     const int ch = (int)(idx - t * p.c4);
@@ -794,7 +794,10 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
         PoolVecArgs v;
         v.g = a, v.c4 = c / 4, v.total = (uint32_t)(total / 4);
         v.div_c4 = FastDiv((uint32_t)v.c4), v.div_ow = FastDiv((uint32_t)a.ow), v.div_oh = FastDiv((uint32_t)a.oh);
-        const unsigned vb = (v.total + 255u) / 256u;
+        // windows of more than 16 taps are long chains of waits: one wave per block there, so that a launch of a few
+        // hundred waves spreads over all CUs (the global 7x7 average at batch 256: 128 blocks of 256 threads before)
+        const unsigned bs = kh * kw > 16 ? 64u : 256u;
+        const unsigned vb = (v.total + bs - 1u) / bs;
         const float4 *x4 = reinterpret_cast<const float4 *>(x);
         float4 *o4 = reinterpret_cast<float4 *>(out);
         // loads kept in flight: the whole window up to 3x3, 16 at a time beyond, 32 when the launch is too small to
@@ -802,7 +805,7 @@ static int pool_common(bool is_max, const float *x, int n, int h, int w, int c, 
         const int taps = kh * kw;
         const int batch_taps = taps <= 4 ? 4 : taps <= 9 ? 9 : (taps <= 16 || v.total > 65536u) ? 16 : 32;
         auto launch = [&](auto kernel) {
-            hipLaunchKernelGGL(kernel, dim3(vb), dim3(256), 0, as_stream(stream), x4, o4, out_packed, v);
+            hipLaunchKernelGGL(kernel, dim3(vb), dim3(bs), 0, as_stream(stream), x4, o4, out_packed, v);
         };
 #define DAB_POOL_LAUNCH(MAX, SIGN)                                               \
     switch (batch_taps) {                                                        \
