@@ -6,11 +6,13 @@
 // 64 output channels.  It multiplies like the plain float convolution (implicit GEMM, rows = pixels, depth = (kh, kw,
 // c), two LDS buffers of SK-deep slices, v_mfma_f32_16x16x4_f32; eight waves as 4 x 2, a wave holds 112 pixels x 32
 // channels), leaves the band in LDS and pools it there.  A pooled row 2*py-1 .. 2*py+1 lies inside the band for all
-// but the band's first pooled row, which also needs the last row of the band above: every block writes the
-// horizontal maxima of its last row to a carry buffer, and a second, small kernel folds the carry of the band above
-// into the first pooled row of each band (a maximum does not depend on the order of its operands).  With the pooled
-// tensor the kernels can write its sign bits, the packed input of the binary convolution that follows
-// (dabnn/bitpack.h:277-293).
+// but the band's first pooled row, which also needs the last row of the band above.  A block is persistent and makes
+// consecutive bands of an image, so the horizontal maxima of a band's last row wait in the registers of the threads
+// that pool the same columns of the next band.  Where another block made the band above (the first band of a
+// block's range; every band when there are several 64-channel tiles), that block writes the row to a carry buffer,
+// and a second, small kernel folds it into the first pooled row of the band below (a maximum does not depend on the
+// order of its operands).  With the pooled tensor the kernels can write its sign bits, the packed input of the
+// binary convolution that follows (dabnn/bitpack.h:277-293).
 #include <float.h>
 
 #include <type_traits>
