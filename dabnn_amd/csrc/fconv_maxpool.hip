@@ -682,8 +682,11 @@ extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, con
         ca.div_c4 = FastDiv((uint32_t)ca.c4), ca.div_pw = FastDiv((uint32_t)b.pw), ca.div_bm1 = FastDiv((uint32_t)(b.bands - 1));
         ca.div_bands = FastDiv((uint32_t)b.bands);
         const unsigned blocks = (unsigned)((total + 255) / 256);
-        if (total == 0) {
-            // one block made every band
+        bool any = !a.chained && total > 0;
+        for (unsigned blk = 1; a.chained && !any && blk < grid.x; ++blk)
+            any = (blk * (long long)a.per + (blk < (unsigned)a.extra ? blk : a.extra)) % b.bands != 0;
+        if (!any) {
+            // every block's range starts with an image's first band (one block, or whole images per block)
         } else if (pooled_packed)
             hipLaunchKernelGGL(maxpool_carry_kernel<true>, dim3(blocks), dim3(256), 0, s, ca);
         else
