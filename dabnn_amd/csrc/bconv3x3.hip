@@ -366,13 +366,25 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
+// Which kernel runs a problem of `tiles` 64-pixel tiles: 0 = the small-problem kernel (blocks split the depth),
+// 1 = the unit kernel at its wide residency, 2 = its NARROW build (64 and 128 input channels only).
+constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2;
+static int pick_build(long long tiles, int cin, int cout) {
+    if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
+    if (cin <= 128) {
+        // four (eight) units or more per wave at four waves per SIMD
+        const long long units = tiles * (cout / 8);
+        if (units >= (cin == 64 ? 4ll : 8ll) * simd_count() * 4) return kBuildNarrow;
+    }
+    return kBuildWide;
+}
+
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
-    if (splits_depth(tiles, CW * 64, a.cout)) return launch_ksplit<CW, MODE>(a, tiles, stream);
+    const int build = pick_build(tiles, CW * 64, a.cout);
+    if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
     if constexpr (CW <= 2) {
-        // four (eight) units or more per wave at four waves per SIMD
-        const long long units = tiles * (a.cout / UnitChannels<CW>::value);
-        if (units >= (CW == 1 ? 4ll : 8ll) * simd_count() * 4) return launch_variant<CW, MODE, true>(a, tiles, stream);
+        if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
     }
     return launch_variant<CW, MODE, false>(a, tiles, stream);
 }
@@ -462,4 +474,9 @@ extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int
 extern "C" int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout) {
     if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return 0;
     return dab::splits_depth((n_out_pixels + 63) / 64, cin, cout) ? 1 : 0;
+}
+
+extern "C" int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout) {
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return -1;
+    return dab::pick_build((n_out_pixels + 63) / 64, cin, cout);
 }

@@ -145,6 +145,15 @@ DAB_API int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int w,
 DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
 
 /*
+ * No counterpart in the reference: which of the three builds of the direct kernel dab_bconv3x3* runs for a problem of
+ * n_out_pixels = N*OH*OW on the current device: 0 = the small-problem kernel (a block splits the depth over its
+ * waves), 1 = the unit kernel at its wide residency, 2 = its four-waves-per-SIMD build (64 and 128 input channels,
+ * many units per wave); -1 for shapes the direct kernel does not take.  For tests and tuning: a parity test names the
+ * build it means to cover.
+ */
+DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
+
+/*
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in

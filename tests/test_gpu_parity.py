@@ -256,6 +256,50 @@ def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, str
     np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
 
 
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,build", [
+    # the four-waves-per-SIMD build of the unit kernel (many units per wave): 128 input channels from 8 units per wave
+    # on, 64 input channels from 4 -- the stage-2 and stage-1 blocks of Bi-Real-18 at batch 256
+    (170, 28, 28, 128, 128, 1, 2), (44, 56, 56, 64, 64, 1, 2),
+    # just below the switch: the wide build on nearly the same problem
+    (160, 28, 28, 128, 128, 1, 1),
+])
+def test_fused_epilogues_of_the_named_build(dab, n, h, w, cin, cout, stride, build):
+    """BinConv + Affine + Add (+ sign) through the build the test names (asked from the library, so the case cannot
+    drift to another kernel unnoticed): images 0, the middle one and the last against the three reference layers
+    bit for bit, the whole batch against the counts-only kernel followed by the separate Affine, Add and pack_mat."""
+    from dabnn_amd import capi
+    oh = (h + 2 - 3) // stride + 1
+    assert capi.lib.dab_bconv3x3_build(n * oh * oh, cin, cout) == build
+    r = rng(26)
+    cw = cin // 64
+    x = r.integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    a[::5] = 0.0
+    b[::10] = 0.0
+    sc = r.standard_normal((n, oh, oh, cout)).astype(np.float32)
+    sc[:, :, :, ::10] = 0.0
+    xd, wd, ad, bd, scd = dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), dev_f(sc)
+    sep = dab.bconv_3x3(xd, wd, stride, 1)
+    dab.affine_inplace(sep, ad, bd)
+    dab.add_inplace(sep, scd)
+    got1 = dab.bconv_3x3_affine_add(xd, wd, ad, bd, scd, stride, 1)
+    got2, packed = dab.bconv_3x3_affine_add_sign(xd, wd, ad, bd, scd, stride, 1)
+    assert torch.equal(got1, sep)
+    assert torch.equal(got2, sep)
+    assert torch.equal(packed, dab.pack_mat(sep))
+    nosc = dab.bconv_3x3_affine_add(xd, wd, ad, bd, None, stride, 1)
+    for i in (0, n // 2 - 2, n - 1):
+        want = orc.baseline_bconv(x[i], wgt, 3, 3, 1, 1, stride, stride)
+        orc.affine_inplace(want, a, b)
+        np.testing.assert_array_equal(nosc[i].cpu().numpy(), want)
+        want = want + sc[i]
+        np.testing.assert_array_equal(got1[i].cpu().numpy(), want)
+        np.testing.assert_array_equal(got2[i].cpu().numpy(), want)
+        np.testing.assert_array_equal(host_u(packed[i]), orc.pack_mat(want))
+
+
 def test_bconv_3x3_unsupported_and_invalid(dab):
     from dabnn_amd.capi import DabUnsupported
     x = torch.zeros((1, 4, 4, 3), dtype=torch.int64, device="cuda")  # 192 channels

@@ -158,18 +158,20 @@ def test_optimize_flag_gives_identical_outputs(mods):
     np.testing.assert_array_equal(outs[0], outs[1])
 
 
+@pytest.mark.parametrize("batch", [1, 2])
 @pytest.mark.parametrize("stem", [False, True])
-def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
+def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem, batch):
+    """Bi-Real-18 as the benchmark runs it at batch 1 (and at 2, the same kernels on two images)."""
     df, models, net = mods
     layers, inits, inputs = models.bireal18(11, stem=stem)
     path = tmp_path / "bireal18.dab"
     path.write_bytes(df.write_model(layers, inits, inputs))
-    x = np.random.default_rng(8).standard_normal((2, 224, 224, 3)).astype(np.float32)
-    n = net.Net(batch=2).read(str(path))
+    x = np.random.default_rng(8).standard_normal((batch, 224, 224, 3)).astype(np.float32)
+    n = net.Net(batch=batch).read(str(path))
     assert sum("Bin Conv" in d for d in n.layers()) == 16
     n.run(x)
-    logits = n.get_blob("logits").reshape(2, -1)
-    assert logits.shape == (2, 1000)
+    logits = n.get_blob("logits").reshape(batch, -1)
+    assert logits.shape == (batch, 1000)
     descs = n.layers()
     # the max pool and every block hand their successor the packed input (at this batch the blocks with 512 input
     # channels run the small-problem kernel, whose work items are whole bytes of sign bits); the three Adds of the
@@ -178,7 +180,7 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem):
     assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
     # the three shortcut branches pool inside their 1x1 convolution; only the global pool is left as a layer
     assert sum("AvePool 2x2 of" in d for d in descs) == 3 and sum(d.startswith("AvePool") for d in descs) == 1
-    for i in range(2):
+    for i in range(batch):
         assert check_every_segment(n, layers, inits, i) >= 20
         assert check_packed_inputs(n, layers, i) == 16
     cpu = orc_net.run_model(layers, inits, x[0])
@@ -231,6 +233,60 @@ def test_bireal18_stem_and_maxpool_in_one_pass(mods, stem):
         want = orc.max_pool(conv[i], 3, 3, 1, 1, 2, 2)
         close(pooled[i], want)
     plain.close()
+
+
+class CachedBlobs:
+    """A Net whose get_blob copies each blob from the device once: at batch 256 a blob is up to 205 MB and the segment
+    checks ask for the same ones many times."""
+
+    def __init__(self, n):
+        self.n, self.cache = n, {}
+
+    def get_blob(self, name):
+        if name not in self.cache:
+            self.cache[name] = self.n.get_blob(name)
+        return self.cache[name]
+
+    def __getattr__(self, attr):
+        return getattr(self.n, attr)
+
+
+@pytest.mark.parametrize("stem", [False, True])
+def test_bireal18_batch256_matches_cpu(mods, stem):
+    """The benchmark's throughput configuration, both stems: at batch 256 other kernels run than at batch 2 or 64 (the
+    four-waves-per-SIMD builds of the direct convolution with their epilogues, 64 x 256 tiles in the pooled shortcut
+    convolutions, the one-pass stem without a carry launch, blocks with 512 input channels that leave the packing to
+    their successor).  Every layer group of the first and the last image against the CPU layers fed with the device's
+    own blobs, and every packed BinConv input against pack_mat of the blob it stands for."""
+    import torch
+    df, models, net = mods
+    from dabnn_amd import capi
+    layers, inits, inputs = models.bireal18(14, stem=stem)
+    batch = 256
+    n = net.Net(batch=batch).read_buf(df.write_model(layers, inits, inputs))
+    descs = n.layers()
+    assert sum("Bin Conv" in d for d in descs) == 16
+    assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == 1
+    # the builds this configuration is there to cover
+    assert capi.lib.dab_bconv3x3_build(batch * 56 * 56, 64, 64) == 2
+    assert capi.lib.dab_bconv3x3_build(batch * 28 * 28, 128, 128) == 2
+    assert capi.lib.dab_bconv3x3_build(batch * 14 * 14, 256, 256) == 1
+    gone = blobs_not_produced(n, layers)
+    gen = torch.Generator().manual_seed(21)
+    x = torch.randn((batch, 224, 224, 3), generator=gen).cuda()
+    n.run(x)
+    cached = CachedBlobs(n)
+    for i in (0, batch - 1):
+        assert check_every_segment(cached, layers, inits, i, gone) >= 19
+        assert check_packed_inputs(cached, layers, i) == 16
+    first = cached.get_blob("logits").reshape(batch, -1).copy()
+    cached.cache.clear()
+    # a second and a third run (the third is the captured graph) give the same logits
+    n.run(x)
+    n.run(x)
+    np.testing.assert_array_equal(n.get_blob("logits").reshape(batch, -1), first)
+    drift_ok(first[0], orc_net.run_model(layers, inits, x[0].cpu().numpy())["logits"])
+    n.close()
 
 
 def test_stem_fusion_leaves_other_graphs_alone(mods):
