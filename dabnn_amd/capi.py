@@ -55,6 +55,7 @@ SIGNATURES = {
     "dab_bconv3x3_affine_add_sign": (_i, [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "dab_binconv_workspace_bytes": (_sz, [_i] * 10),
     "dab_binconv_forward": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 8 + [_vp, _vp, _sz, ctypes.POINTER(_i), _vp]),
+    "dab_binconv_forward_static": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 8 + [_vp, ctypes.POINTER(_i), _vp]),
     "dab_fconv": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 9 + [_vp, _vp]),
     "dab_fconv_affine_relu": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp] + [_i] * 10 + [_vp, _vp]),
     "dab_ave_pool2_fconv1x1": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),

@@ -2,9 +2,37 @@
 // binarise the fp32 input and run the binary convolution, choosing between
 // the direct 3x3 kernel and im2col + bgemm the way BinConv::method() (:80-98)
 // does on the reference's optimised targets.
+#include <mutex>
+
 #include "common.h"
 
 namespace dab {
+
+// Scratch of dab_binconv_forward_static: the packed activations (direct arm) or the column matrix (bgemm arm) of one
+// call.  One copy per GPU, held until the process ends; the array's name is only a handle for hipGetSymbolAddress in
+// host code, the kernels get the device address that call returns.
+static __device__ __align__(256) unsigned char scratch[DAB_BINCONV_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+static void *scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, resolved on the first call there
+static std::mutex scratch_mutex;
+
+// Device address of this GPU's copy of `scratch` (the current device's).
+static int static_scratch(void **out) {
+    int dev = 0;
+    DAB_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(DAB_EUNSUPPORTED, "dab_binconv_forward_static: device index %d", dev);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        DAB_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (p == nullptr) return fail(DAB_EHIP, "dab_binconv_forward_static: no device address for the scratch array");
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return DAB_OK;
+}
+
 int fill_f32(float *x, long long total, float v, hipStream_t s);
 
 static bool direct_ok(int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int cout) {
@@ -63,4 +91,25 @@ extern "C" int dab_binconv_forward(const float *x, int n, int h, int w, int c, c
     rc = dab_bgemm(cout, (int)npix, hwc_words, wgt_t, cout, col, row_words, out, cout, stream);
     if (rc == DAB_OK && method_out) *method_out = 1;
     return rc;
+}
+
+extern "C" int dab_binconv_forward_static(const float *x, int n, int h, int w, int c, const uint64_t *wgt,
+                                          const uint64_t *wgt_t, int hwc_words, int kh, int kw, int pad_h, int pad_w,
+                                          int stride_h, int stride_w, int cout, float *out, int *method_out,
+                                          dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && kh > 0 && kw > 0 && stride_h > 0 && stride_w > 0,
+                "dab_binconv_forward_static: non-positive dimension");
+    const size_t need = dab_binconv_workspace_bytes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w);
+    if (need > (size_t)DAB_BINCONV_STATIC_SCRATCH_BYTES)
+        return fail(DAB_EUNSUPPORTED,
+                    "dab_binconv_forward_static: this problem needs %zu bytes of scratch, the static buffer holds %zu; "
+                    "use dab_binconv_forward with a workspace of your own",
+                    need, (size_t)DAB_BINCONV_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != DAB_OK) return rc;
+    // both arms overwrite every word of the scratch they read, so nothing of the previous call has to be cleared
+    return dab_binconv_forward(x, n, h, w, c, wgt, wgt_t, hwc_words, kh, kw, pad_h, pad_w, stride_h, stride_w, cout, out,
+                               ws, (size_t)DAB_BINCONV_STATIC_SCRATCH_BYTES, method_out, stream);
 }

@@ -170,6 +170,22 @@ DAB_API int dab_binconv_forward(const float *x, int n, int h, int w, int c, cons
                         int hwc_words, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int cout,
                         float *out, void *workspace, size_t workspace_bytes, int *method_out, dab_stream_t stream);
 
+/*
+ * No counterpart in the reference.  dab_binconv_forward for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the workspace is a buffer of
+ * DAB_BINCONV_STATIC_SCRATCH_BYTES that lives inside the library's code object, one copy per GPU, held until the
+ * process ends.  Same arguments, results and error codes as dab_binconv_forward without the workspace pair; problems
+ * whose dab_binconv_workspace_bytes(...) exceeds the buffer return DAB_EUNSUPPORTED.  The call allocates and frees
+ * nothing on the device.  All calls on one GPU share that GPU's buffer: two calls that overlap in time on the same
+ * GPU (different streams or threads) race; calls on one stream are ordered and safe.  The first call on a device
+ * resolves the buffer's address (hipGetSymbolAddress); make it outside a graph capture.
+ */
+#define DAB_BINCONV_STATIC_SCRATCH_BYTES (16u << 20)
+DAB_API int dab_binconv_forward_static(const float *x, int n, int h, int w, int c, const uint64_t *wgt,
+                                       const uint64_t *wgt_t, int hwc_words, int kh, int kw, int pad_h, int pad_w,
+                                       int stride_h, int stride_w, int cout, float *out, int *method_out,
+                                       dab_stream_t stream);
+
 /* ------------------------------------------------------------------ float glue */
 
 /*
