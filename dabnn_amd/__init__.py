@@ -31,5 +31,7 @@ from .ops import (  # noqa: F401
     pad,
     prelu_inplace,
     relu_inplace,
+    shuffle_bit_inplace,
+    split_bit,
     weight_transpose,
 )

@@ -46,6 +46,8 @@ SIGNATURES = {
     "dab_bitpack_nhwc": (_i, [_vp, _vp, _i64, _i, _vp]),
     "dab_bitpack_nchw": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "dab_pad_bit": (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp]),
+    "dab_split_bit": (_i, [_vp, _i64, _i, _vp, _vp, _vp]),
+    "dab_shuffle_bit_inplace": (_i, [_vp, _i64, _i, _vp]),
     "dab_fused_binarize_im2col": (_i, [_vp] + [_i] * 12 + [_vp, _vp]),
     "dab_col_row_words": (_i, [_i, _i, _i]),
     "dab_bgemm": (_i, [_i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp]),

@@ -91,6 +91,46 @@ __global__ __launch_bounds__(256) void weight_transpose_kernel(const uint64_t *_
     wt[idx] = w[(size_t)j * k + i];
 }
 
+// Split::forward_impl (dabnn/layers/Split.cpp:6-21): word j of pixel p goes to out1[p][j] for j < cw/2, else to
+// out2[p][j - cw/2].  One thread per input word, coalesced reads.
+__global__ __launch_bounds__(256) void split_bit_kernel(const uint64_t *__restrict__ x, uint64_t *__restrict__ out1,
+                                                        uint64_t *__restrict__ out2, long long n_pix, int cw) {
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n_pix * cw) return;
+    const long long pix = idx / cw;
+    const int j = (int)(idx - pix * cw), half = cw / 2;
+    const uint64_t v = x[idx];
+    if (j < half)
+        out1[pix * half + j] = v;
+    else
+        out2[pix * half + j - half] = v;
+}
+
+// Shuffle::forward_impl (dabnn/layers/Shuffle.cpp:6-43), one thread per pixel, in place:
+//   128 channels: the pixel's four 32-bit quarters a b c d become a c b d
+//   256 channels: words 1 and 2 change places;  512 channels: words 2,3 change places with words 4,5
+//   any other channel count is left as it is, as in the reference
+__global__ __launch_bounds__(256) void shuffle_bit_kernel(uint64_t *__restrict__ x, long long n_pix, int elem_c) {
+    const long long pix = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (pix >= n_pix) return;
+    if (elem_c == 128) {
+        uint64_t *p = x + pix * 2;
+        const uint64_t w0 = p[0], w1 = p[1];
+        p[0] = (w0 & 0xffffffffull) | (w1 << 32);
+        p[1] = (w0 >> 32) | (w1 & 0xffffffff00000000ull);
+    } else if (elem_c == 256) {
+        uint64_t *p = x + pix * 4;
+        const uint64_t t = p[1];
+        p[1] = p[2];
+        p[2] = t;
+    } else if (elem_c == 512) {
+        uint64_t *p = x + pix * 8;
+        const uint64_t t2 = p[2], t3 = p[3];
+        p[2] = p[4], p[3] = p[5];
+        p[4] = t2, p[5] = t3;
+    }
+}
+
 static unsigned blocks_for(long long total, int per_block) {
     long long b = (total + per_block - 1) / per_block;
     return (unsigned)(b < 1 ? 1 : b);
@@ -144,6 +184,32 @@ extern "C" int dab_weight_transpose(const uint64_t *w, int m, int k, uint64_t *w
     DAB_REQUIRE(m > 0 && k > 0, "dab_weight_transpose: m %d k %d", m, k);
     hipLaunchKernelGGL(weight_transpose_kernel, dim3(blocks_for((long long)m * k, 256)), dim3(256), 0, as_stream(stream),
                        w, wt, m, k);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_split_bit(const uint64_t *x, int64_t n_pix, int cw, uint64_t *out1, uint64_t *out2, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x && out1 && out2, "dab_split_bit: null pointer");
+    DAB_REQUIRE(n_pix > 0 && cw > 0, "dab_split_bit: n_pix %lld cw %d", (long long)n_pix, cw);
+    // the reference asserts elem_c % 128 == 0 && elem_c <= 512 (dabnn/layers/Split.h:22-23)
+    DAB_REQUIRE(cw % 2 == 0 && cw <= 8, "Split: %d channels", cw * 64);
+    if (n_pix * cw >= (1ll << 40)) return fail(DAB_EUNSUPPORTED, "dab_split_bit: tensor too large");
+    hipLaunchKernelGGL(split_bit_kernel, dim3(blocks_for((long long)n_pix * cw, 256)), dim3(256), 0, as_stream(stream), x, out1,
+                       out2, (long long)n_pix, cw);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+extern "C" int dab_shuffle_bit_inplace(uint64_t *x, int64_t n_pix, int elem_c, dab_stream_t stream) {
+    using namespace dab;
+    DAB_REQUIRE(x, "dab_shuffle_bit_inplace: null pointer");
+    DAB_REQUIRE(n_pix > 0, "dab_shuffle_bit_inplace: n_pix %lld", (long long)n_pix);
+    // dabnn/layers/Shuffle.h:19-20
+    DAB_REQUIRE(elem_c > 0 && elem_c % 128 == 0 && elem_c <= 512, "Shuffle: %d channels", elem_c);
+    if (n_pix >= (1ll << 40)) return fail(DAB_EUNSUPPORTED, "dab_shuffle_bit_inplace: tensor too large");
+    hipLaunchKernelGGL(shuffle_bit_kernel, dim3(blocks_for((long long)n_pix, 256)), dim3(256), 0, as_stream(stream), x,
+                       (long long)n_pix, elem_c);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }

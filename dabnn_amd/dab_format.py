@@ -59,7 +59,8 @@ class Builder:
     Offsets handed out are distances from the END of the finished buffer, as in
     the official builders."""
 
-    def __init__(self):
+    def __init__(self, trim_vtables=False):
+        self.trim_vtables = trim_vtables  # drop trailing absent slots from every vtable, as flatc's builders do
         self.chunks = []  # in prepend order
         self.size = 0
         self.minalign = 1
@@ -123,6 +124,10 @@ class Builder:
         vt = [4 + 2 * n_slots, table_off - table_end]
         for slot in range(n_slots):
             vt.append(table_off - positions[slot] if slot in positions else 0)
+        if self.trim_vtables:
+            while len(vt) > 2 and vt[-1] == 0:
+                vt.pop()
+            vt[0] = 2 * len(vt)
         vt_bytes = struct.pack("<%dH" % len(vt), *vt)
         if vt_bytes in self.vtables:
             vt_off = self.vtables[vt_bytes]
@@ -175,11 +180,13 @@ def _param_table(b, ltype, params):
     return b.table(len(spec), fields)
 
 
-def write_model(layers, initializers, inputs, version=MODEL_VERSION):
+def write_model(layers, initializers, inputs, version=MODEL_VERSION, trim_vtables=False):
     """layers: list of dicts {"type": str, "name": str, **params};
     initializers: list of dicts {"name", "shape", "data" (np.float32 or np.uint64 array), "align_hwc_to_128": bool};
-    inputs: list of (name, shape).  Returns the file content."""
-    b = Builder()
+    inputs: list of (name, shape).  Returns the file content.  Scalars at their default (Float32 data, FpConv2D
+    type, align_hwc_to_128 false) are left out and equal vtables are shared, as flatc's builders do; trim_vtables
+    also drops the trailing absent slots of every vtable, their other habit."""
+    b = Builder(trim_vtables)
     layer_offs = []
     for layer in layers:
         ltype = layer["type"]

@@ -13,7 +13,7 @@ namespace bnn {
 
 class Net;
 
-class Layer {
+class BNN_API Layer {
    protected:
     using NetCP = const std::weak_ptr<Net>;
     using MatCP = const std::shared_ptr<Mat>;
@@ -35,12 +35,12 @@ class Layer {
 };
 
 // BNN_ASSERT of the reference throws std::runtime_error (common/helper.h:69-77).
-[[noreturn]] void bnn_fail(const std::string &msg);
+[[noreturn]] BNN_API void bnn_fail(const std::string &msg);
 #define BNN_ASSERT(cond, msg)                    \
     do {                                         \
         if (!(cond)) ::bnn::bnn_fail(msg);       \
     } while (0)
 // A failed C-ABI call becomes the same exception type.
-void dab_check(int rc);
+BNN_API void dab_check(int rc);
 
 }  // namespace bnn

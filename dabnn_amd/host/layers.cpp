@@ -17,7 +17,7 @@ void dab_check(int rc) {
 // ---------------------------------------------------------------- Layer
 Layer::~Layer() {}
 
-Layer::MatP Layer::mat(const std::string &name) const { return net_.lock()->get_blob(name); }
+Layer::MatP Layer::mat(const std::string &name) const { return net_.lock()->blob(name); }
 
 void *Layer::stream() const { return net_.lock()->stream(); }
 
@@ -43,7 +43,22 @@ BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad
     BNN_ASSERT(weight_mat->data_type == DataType::Bit, "BinConv weight must be Bit");
     BNN_ASSERT(input_mat->elem_c % 64 == 0, "BinConv needs a multiple of 64 input channels, got " +
                                                 std::to_string(input_mat->elem_c));
-    BNN_ASSERT(weight_mat->total() % weight_mat->n == 0, "weight size is not a multiple of the filter count");
+    BNN_ASSERT(weight_mat->n > 0 && weight_mat->total() % weight_mat->n == 0, "weight size is not a multiple of the filter count");
+    // the kernels take every extent from the input and the filter count: a weight tensor that is shorter than that
+    // geometry says would be read past its end
+    BNN_ASSERT(weight_mat->elem_c == input_mat->elem_c, "BinConv weight has " + std::to_string(weight_mat->elem_c) +
+                                                            " input channels, the input blob " + std::to_string(input_mat->elem_c));
+    {
+        const size_t per = weight_mat->total() / weight_mat->n;
+        const size_t bits = (size_t)kernel_h() * kernel_w() * input_mat->elem_c;
+        BNN_ASSERT(per * 64 >= bits && per <= (size_t)dab_col_row_words(kernel_h(), kernel_w(), input_mat->elem_c),
+                   "BinConv weight holds " + std::to_string(per) + " words per filter, its geometry needs " +
+                       std::to_string((bits + 63) / 64));
+        if (direct_conv_compatible())
+            BNN_ASSERT(per == (size_t)9 * (input_mat->elem_c / 64), "BinConv weight holds " + std::to_string(per) +
+                                                                        " words per filter, the direct 3x3 kernel walks " +
+                                                                        std::to_string(9 * (input_mat->elem_c / 64)));
+    }
 
     const std::string binarized_name = "binaized_for_" + output + "_cal";
     if (!n->has_blob(binarized_name))
@@ -62,8 +77,8 @@ BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad
     const int m = weight_mat->n;
     const int k = (int)(weight_mat->total() / m);
     transposed_weight_mat = std::make_shared<Mat>((size_t)m * k, DataType::Bit, "trans_" + weight);
-    dab_check(dab_weight_transpose(static_cast<const uint64_t *>(weight_mat->data), m, k,
-                                   static_cast<uint64_t *>(transposed_weight_mat->data), n->stream()));
+    dab_check(dab_weight_transpose(static_cast<const uint64_t *>(weight_mat->dev), m, k,
+                                   static_cast<uint64_t *>(transposed_weight_mat->dev), n->stream()));
     n->add_mat("trans_" + weight, transposed_weight_mat);
 }
 
@@ -81,27 +96,27 @@ BinConv::Method BinConv::method() const {
 
 void BinConv::forward_impl() const {
     void *s = stream();
-    const auto *x = static_cast<const float *>(input_mat->data);
-    auto *out = static_cast<float *>(output_mat->data);
+    const auto *x = static_cast<const float *>(input_mat->dev);
+    auto *out = static_cast<float *>(output_mat->dev);
     const int n = input_mat->n, h = input_mat->h, w = input_mat->w, c = input_mat->elem_c;
     switch (method()) {
         case DIRECT_CONV: {
             // pack_mat + (pad +) bconv_3x3, dabnn/layers/BinConv.cpp:146-150
-            auto *packed = static_cast<uint64_t *>(binarized_mat->data);
+            auto *packed = static_cast<uint64_t *>(binarized_mat->dev);
             if (!input_prepacked) dab_check(dab_bitpack_nhwc(x, packed, (int64_t)n * h * w, c, s));
             if (fused_a && fused_sign_out) {
                 dab_check(dab_bconv3x3_affine_add_sign(
-                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n, stride_h, pad_h,
-                    static_cast<const float *>(fused_a->data), static_cast<const float *>(fused_b->data),
-                    fused_shortcut ? static_cast<const float *>(fused_shortcut->data) : nullptr, out,
-                    static_cast<uint64_t *>(fused_sign_out->data), s));
+                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->dev), weight_mat->n, stride_h, pad_h,
+                    static_cast<const float *>(fused_a->dev), static_cast<const float *>(fused_b->dev),
+                    fused_shortcut ? static_cast<const float *>(fused_shortcut->dev) : nullptr, out,
+                    static_cast<uint64_t *>(fused_sign_out->dev), s));
             } else if (fused_a) {
                 dab_check(dab_bconv3x3_affine_add(
-                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n, stride_h, pad_h,
-                    static_cast<const float *>(fused_a->data), static_cast<const float *>(fused_b->data),
-                    fused_shortcut ? static_cast<const float *>(fused_shortcut->data) : nullptr, out, s));
+                    packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->dev), weight_mat->n, stride_h, pad_h,
+                    static_cast<const float *>(fused_a->dev), static_cast<const float *>(fused_b->dev),
+                    fused_shortcut ? static_cast<const float *>(fused_shortcut->dev) : nullptr, out, s));
             } else {
-                dab_check(dab_bconv3x3(packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->data), weight_mat->n,
+                dab_check(dab_bconv3x3(packed, n, h, w, c, static_cast<const uint64_t *>(weight_mat->dev), weight_mat->n,
                                        stride_h, pad_h, out, s));
             }
             break;
@@ -109,14 +124,14 @@ void BinConv::forward_impl() const {
         case BGEMM: {
             // fill + fused_binarize_im2col + bgemm, dabnn/layers/BinConv.cpp:152-165
             dab_check(dab_fill_f32(out, (int64_t)output_mat->total(), 0.f, s));
-            auto *col = static_cast<uint64_t *>(col_mat->data);
+            auto *col = static_cast<uint64_t *>(col_mat->dev);
             dab_check(dab_fused_binarize_im2col(x, n, h, w, c, kernel_h(), kernel_w(), pad_h, pad_w, stride_h, stride_w, 1,
                                                 1, col, s));
             const int m = weight_mat->n;
             const int cols = n * output_mat->h * output_mat->w;
             const int k = (int)(weight_mat->total() / m);
             const int ldb = dab_col_row_words(kernel_h(), kernel_w(), c);  // rows are padded to 128 bits
-            dab_check(dab_bgemm(m, cols, k, static_cast<const uint64_t *>(transposed_weight_mat->data), m, col, ldb, out, m,
+            dab_check(dab_bgemm(m, cols, k, static_cast<const uint64_t *>(transposed_weight_mat->dev), m, col, ldb, out, m,
                                 s));
             break;
         }
@@ -146,7 +161,9 @@ FloatConv::FloatConv(NetCP net, css name, css input, css weight, css bias, css o
       pad_w(pad_w_),
       stride_h(stride_h_),
       stride_w(stride_w_),
-      dilation(dilation_) {}
+      dilation(dilation_) {
+    check_operands();
+}
 
 FloatConv::FloatConv(NetCP net, css name, css input, css weight, css output, int pad_h_, int pad_w_, int stride_h_,
                      int stride_w_, int dilation_)
@@ -158,36 +175,50 @@ FloatConv::FloatConv(NetCP net, css name, css input, css weight, css output, int
       pad_w(pad_w_),
       stride_h(stride_h_),
       stride_w(stride_w_),
-      dilation(dilation_) {}
+      dilation(dilation_) {
+    check_operands();
+}
+
+// The kernel sizes its weight descriptor as cout * kh * kw * input channels: the tensors must say the same.
+void FloatConv::check_operands() const {
+    BNN_ASSERT(input_mat->data_type == DataType::Float && weight_mat->data_type == DataType::Float, "FloatConv operands must be float");
+    BNN_ASSERT(weight_mat->c == input_mat->c, "FloatConv weight has " + std::to_string(weight_mat->c) +
+                                                  " input channels, the input blob " + std::to_string(input_mat->c));
+    BNN_ASSERT(weight_mat->total() == (size_t)weight_mat->n * weight_mat->h * weight_mat->w * input_mat->c,
+               "FloatConv weight does not match its shape");
+    BNN_ASSERT(output_mat->c == weight_mat->n, "FloatConv output does not have one channel per filter");
+    if (bias_mat) BNN_ASSERT((int)bias_mat->total() == weight_mat->n, "FloatConv bias does not match the filter count");
+    BNN_ASSERT(stride_h > 0 && stride_w > 0 && dilation > 0 && pad_h >= 0 && pad_w >= 0, "FloatConv: bad stride, dilation or pad");
+}
 
 void FloatConv::forward_impl() const {
     if (fused_pool_input) {
         dab_check(dab_ave_pool2_fconv1x1(
-            static_cast<const float *>(fused_pool_input->data), fused_pool_input->n, fused_pool_input->h, fused_pool_input->w,
-            fused_pool_input->c, static_cast<const float *>(weight_mat->data),
-            bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
-            fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
-            fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, output_mat->c,
-            static_cast<float *>(input_mat->data), static_cast<float *>(output_mat->data), stream()));
+            static_cast<const float *>(fused_pool_input->dev), fused_pool_input->n, fused_pool_input->h, fused_pool_input->w,
+            fused_pool_input->c, static_cast<const float *>(weight_mat->dev),
+            bias_mat ? static_cast<const float *>(bias_mat->dev) : nullptr,
+            fused_a ? static_cast<const float *>(fused_a->dev) : nullptr,
+            fused_b ? static_cast<const float *>(fused_b->dev) : nullptr, fused_relu ? 1 : 0, output_mat->c,
+            static_cast<float *>(input_mat->dev), static_cast<float *>(output_mat->dev), stream()));
         return;
     }
     if (fused_maxpool_out) {
         dab_check(dab_fconv_maxpool(
-            static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
-            static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
-            fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
-            fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
-            pad_h, pad_w, stride_h, stride_w, dilation, dilation, weight_mat->n, static_cast<float *>(fused_maxpool_out->data),
-            fused_maxpool_sign ? static_cast<uint64_t *>(fused_maxpool_sign->data) : nullptr,
-            static_cast<float *>(fused_maxpool_carry->data), stream()));
+            static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
+            static_cast<const float *>(weight_mat->dev), bias_mat ? static_cast<const float *>(bias_mat->dev) : nullptr,
+            fused_a ? static_cast<const float *>(fused_a->dev) : nullptr,
+            fused_b ? static_cast<const float *>(fused_b->dev) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
+            pad_h, pad_w, stride_h, stride_w, dilation, dilation, weight_mat->n, static_cast<float *>(fused_maxpool_out->dev),
+            fused_maxpool_sign ? static_cast<uint64_t *>(fused_maxpool_sign->dev) : nullptr,
+            static_cast<float *>(fused_maxpool_carry->dev), stream()));
         return;
     }
     dab_check(dab_fconv_affine_relu(
-        static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
-        static_cast<const float *>(weight_mat->data), bias_mat ? static_cast<const float *>(bias_mat->data) : nullptr,
-        fused_a ? static_cast<const float *>(fused_a->data) : nullptr,
-        fused_b ? static_cast<const float *>(fused_b->data) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
-        pad_h, pad_w, stride_h, stride_w, dilation, dilation, output_mat->c, static_cast<float *>(output_mat->data),
+        static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w, input_mat->c,
+        static_cast<const float *>(weight_mat->dev), bias_mat ? static_cast<const float *>(bias_mat->dev) : nullptr,
+        fused_a ? static_cast<const float *>(fused_a->dev) : nullptr,
+        fused_b ? static_cast<const float *>(fused_b->dev) : nullptr, fused_relu ? 1 : 0, weight_mat->h, weight_mat->w,
+        pad_h, pad_w, stride_h, stride_w, dilation, dilation, output_mat->c, static_cast<float *>(output_mat->dev),
         stream()));
 }
 
@@ -210,9 +241,9 @@ Affine::Affine(NetCP net, css name, css data, css a, css b)
 }
 
 void Affine::forward_impl() const {
-    dab_check(dab_affine_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->n * data_mat->h * data_mat->w,
-                                 data_mat->c, static_cast<const float *>(a_mat->data),
-                                 static_cast<const float *>(b_mat->data), stream()));
+    dab_check(dab_affine_inplace(static_cast<float *>(data_mat->dev), (int64_t)data_mat->n * data_mat->h * data_mat->w,
+                                 data_mat->c, static_cast<const float *>(a_mat->dev),
+                                 static_cast<const float *>(b_mat->dev), stream()));
 }
 
 Add::Add(NetCP net, css name, css input1, css input2)
@@ -221,14 +252,14 @@ Add::Add(NetCP net, css name, css input1, css input2)
 }
 
 void Add::forward_impl() const {
-    dab_check(dab_add_inplace(static_cast<float *>(input1_mat->data), static_cast<const float *>(input2_mat->data),
+    dab_check(dab_add_inplace(static_cast<float *>(input1_mat->dev), static_cast<const float *>(input2_mat->dev),
                               (int64_t)input1_mat->total(), stream()));
 }
 
 Relu::Relu(NetCP net, css name, css data) : Layer(net, name, "Relu"), data_mat(mat(data)) {}
 
 void Relu::forward_impl() const {
-    dab_check(dab_relu_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->total(), stream()));
+    dab_check(dab_relu_inplace(static_cast<float *>(data_mat->dev), (int64_t)data_mat->total(), stream()));
 }
 
 // dabnn/layers/PRelu.cpp:6-30; the size check is the reference's, made once at construction
@@ -239,8 +270,8 @@ PRelu::PRelu(NetCP net, css name, css data, css slope)
 }
 
 void PRelu::forward_impl() const {
-    dab_check(dab_prelu_inplace(static_cast<float *>(data_mat->data), (int64_t)data_mat->n * data_mat->h * data_mat->w,
-                                data_mat->c, static_cast<const float *>(slope_mat->data), (int)slope_mat->total(), stream()));
+    dab_check(dab_prelu_inplace(static_cast<float *>(data_mat->dev), (int64_t)data_mat->n * data_mat->h * data_mat->w,
+                                data_mat->c, static_cast<const float *>(slope_mat->dev), (int)slope_mat->total(), stream()));
 }
 
 // dabnn/layers/Concat.cpp:7-21 (two inputs, channel axis)
@@ -252,10 +283,35 @@ Concat::Concat(NetCP net, css name, css input1, css input2, css output)
 }
 
 void Concat::forward_impl() const {
-    dab_check(dab_concat_channels(static_cast<const float *>(input1_mat->data), input1_mat->c,
-                                  static_cast<const float *>(input2_mat->data), input2_mat->c,
+    dab_check(dab_concat_channels(static_cast<const float *>(input1_mat->dev), input1_mat->c,
+                                  static_cast<const float *>(input2_mat->dev), input2_mat->c,
                                   (int64_t)input1_mat->n * input1_mat->h * input1_mat->w,
-                                  static_cast<float *>(output_mat->data), stream()));
+                                  static_cast<float *>(output_mat->dev), stream()));
+}
+
+// ---------------------------------------------------------------- Split / Shuffle (Bit blobs)
+Split::Split(NetCP net, css name, css input, css output1, css output2)
+    : Layer(net, name, "Split"), input_mat(mat(input)), output_mat1(mat(output1)), output_mat2(mat(output2)) {
+    BNN_ASSERT(input_mat->data_type == DataType::Bit, "Split only supports bit mat");  // dabnn/layers/Split.h:19-23
+    BNN_ASSERT(input_mat->elem_c % 128 == 0 && input_mat->elem_c <= 512, "Split: " + std::to_string(input_mat->elem_c) + " channels");
+    BNN_ASSERT(output_mat1->data_type == DataType::Bit && output_mat2->data_type == DataType::Bit &&
+                   output_mat1->total() * 2 == input_mat->total() && output_mat2->total() * 2 == input_mat->total(),
+               "Split outputs must each hold half of the input's words");
+}
+
+void Split::forward_impl() const {
+    dab_check(dab_split_bit(static_cast<const uint64_t *>(input_mat->dev), (int64_t)(input_mat->total() / input_mat->c), input_mat->c,
+                            static_cast<uint64_t *>(output_mat1->dev), static_cast<uint64_t *>(output_mat2->dev), stream()));
+}
+
+Shuffle::Shuffle(NetCP net, css name, css data) : Layer(net, name, "Shuffle"), data_mat(mat(data)) {
+    BNN_ASSERT(data_mat->data_type == DataType::Bit, "Shuffle only supports bit mat");  // dabnn/layers/Shuffle.h:16-20
+    BNN_ASSERT(data_mat->elem_c % 128 == 0 && data_mat->elem_c <= 512, "Shuffle: " + std::to_string(data_mat->elem_c) + " channels");
+}
+
+void Shuffle::forward_impl() const {
+    dab_check(dab_shuffle_bit_inplace(static_cast<uint64_t *>(data_mat->dev), (int64_t)(data_mat->total() / data_mat->c),
+                                      data_mat->elem_c, stream()));
 }
 
 // ---------------------------------------------------------------- pooling
@@ -272,9 +328,9 @@ AvePool::AvePool(NetCP net, css name, css input, css output, int kernel_h_, int 
       stride_w(stride_w_) {}
 
 void AvePool::forward_impl() const {
-    dab_check(dab_ave_pool(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+    dab_check(dab_ave_pool(static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w,
                            input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
-                           static_cast<float *>(output_mat->data), stream()));
+                           static_cast<float *>(output_mat->dev), stream()));
 }
 
 MaxPool::MaxPool(NetCP net, css name, css input, css output, int kernel_h_, int kernel_w_, int pad_h_, int pad_w_,
@@ -291,15 +347,15 @@ MaxPool::MaxPool(NetCP net, css name, css input, css output, int kernel_h_, int 
 
 void MaxPool::forward_impl() const {
     if (fused_sign_out) {
-        dab_check(dab_max_pool_sign(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+        dab_check(dab_max_pool_sign(static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w,
                                     input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
-                                    static_cast<float *>(output_mat->data), static_cast<uint64_t *>(fused_sign_out->data),
+                                    static_cast<float *>(output_mat->dev), static_cast<uint64_t *>(fused_sign_out->dev),
                                     stream()));
         return;
     }
-    dab_check(dab_max_pool(static_cast<const float *>(input_mat->data), input_mat->n, input_mat->h, input_mat->w,
+    dab_check(dab_max_pool(static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w,
                            input_mat->c, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w,
-                           static_cast<float *>(output_mat->data), stream()));
+                           static_cast<float *>(output_mat->dev), stream()));
 }
 
 }  // namespace bnn

@@ -1,6 +1,6 @@
-// The layers of the Bi-Real and BiDenseNet paths (dabnn/layers/{BinConv,FloatConv,
-// Affine,Add,AvePool,MaxPool,Relu,PRelu,Concat}.{h,cpp}); constructor signatures
-// follow the reference.
+// The layers Net::prepare of the reference builds (dabnn/layers/{BinConv,FloatConv,
+// Affine,Add,AvePool,MaxPool,Relu,PRelu,Concat,Split,Shuffle}.{h,cpp}); constructor
+// signatures follow the reference.
 #pragma once
 
 #include "layer.h"
@@ -9,7 +9,7 @@ namespace bnn {
 
 using css = const std::string &;
 
-class BinConv : public Layer {
+class BNN_API BinConv : public Layer {
    public:
     MatP input_mat;
     MatP binarized_mat;  // packed input of the direct method
@@ -41,7 +41,7 @@ class BinConv : public Layer {
     bool direct_conv_compatible() const;
 };
 
-class FloatConv : public Layer {
+class BNN_API FloatConv : public Layer {
    public:
     MatP input_mat, weight_mat, bias_mat, output_mat;
     // Affine (and Relu) layers that follow on the output blob, applied in the convolution's epilogue when set
@@ -61,44 +61,63 @@ class FloatConv : public Layer {
               int dilation);
     void forward_impl() const override;
     std::string to_str() const override;
+
+   private:
+    void check_operands() const;
 };
 
-class Affine : public Layer {
+class BNN_API Affine : public Layer {
    public:
     MatP data_mat, a_mat, b_mat;
     Affine(NetCP net, css name, css data, css a, css b);
     void forward_impl() const override;
 };
 
-class Add : public Layer {
+class BNN_API Add : public Layer {
    public:
     MatP input1_mat, input2_mat;
     Add(NetCP net, css name, css input1, css input2);
     void forward_impl() const override;
 };
 
-class Relu : public Layer {
+class BNN_API Relu : public Layer {
    public:
     MatP data_mat;
     Relu(NetCP net, css name, css data);
     void forward_impl() const override;
 };
 
-class PRelu : public Layer {
+class BNN_API PRelu : public Layer {
    public:
     MatP data_mat, slope_mat;
     PRelu(NetCP net, css name, css data, css slope);
     void forward_impl() const override;
 };
 
-class Concat : public Layer {
+class BNN_API Concat : public Layer {
    public:
     MatP input1_mat, input2_mat, output_mat;
     Concat(NetCP net, css name, css input1, css input2, css output);
     void forward_impl() const override;
 };
 
-class AvePool : public Layer {
+// dabnn/layers/Split.{h,cpp}: a Bit blob's words per pixel cut in two halves (first half -> output 1).
+class BNN_API Split : public Layer {
+   public:
+    MatP input_mat, output_mat1, output_mat2;
+    Split(NetCP net, css name, css input, css output1, css output2);
+    void forward_impl() const override;
+};
+
+// dabnn/layers/Shuffle.{h,cpp}: the channel shuffle of a two-group network on packed words, in place.
+class BNN_API Shuffle : public Layer {
+   public:
+    MatP data_mat;
+    Shuffle(NetCP net, css name, css data);
+    void forward_impl() const override;
+};
+
+class BNN_API AvePool : public Layer {
    public:
     MatP input_mat, output_mat;
     const int kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w;
@@ -107,7 +126,7 @@ class AvePool : public Layer {
     void forward_impl() const override;
 };
 
-class MaxPool : public Layer {
+class BNN_API MaxPool : public Layer {
    public:
     MatP input_mat, output_mat;
     // Set by Net::prepare when a direct BinConv reads the pooled blob: its packed input, written in the same pass.

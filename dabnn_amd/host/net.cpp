@@ -9,43 +9,15 @@
 #include <stdexcept>
 
 #include "../../include/dabnn_hip.h"
-#include "flatbuf.h"
 #include "layers.h"
+#include "model.h"
 
 namespace bnn {
 
 namespace {
 
-constexpr uint32_t kModelVersion = 2;  // BNN_LATEST_MODEL_VERSION, common/macros.h:6
-
-// vtable slots of common/dab.fbs (declaration order)
-enum ModelSlot { M_LAYERS = 0, M_INITIALIZERS = 1, M_INPUTS = 2, M_VERSION = 3 };
-enum TensorSlot { T_DATA_TYPE = 0, T_BIN_DATA = 1, T_FLOAT_DATA = 2, T_SHAPE = 3, T_NAME = 4, T_ALIGN = 5 };
-enum InputSlot { I_SHAPE = 0, I_NAME = 1 };
-enum LayerSlot {
-    L_TYPE = 0, L_FPCONV = 1, L_BINCONV = 2, L_AVEPOOL = 3, L_MAXPOOL = 4, L_RELU = 5, L_SOFTMAX = 6, L_FC = 7, L_ADD = 8,
-    L_CONCAT = 9, L_AFFINE = 10, L_BINARIZE = 11, L_SPLIT = 12, L_SHUFFLE = 13, L_NAME = 14, L_PRELU = 15
-};
-enum LayerType {
-    FpConv2D = 0, AvePoolT, MaxPoolT, ReluT, Softmax, FC, AddT, ConcatT, BinConv2D, AffineT, Binarize, Split, Shuffle, PReluT
-};
-const char *kLayerTypeNames[] = {"FpConv2D", "AvePool", "MaxPool", "Relu",     "Softmax", "FC",      "Add",
-                                 "Concat",   "BinConv2D", "Affine", "Binarize", "Split",   "Shuffle", "PRelu"};
-
 void hip_check(hipError_t e, const char *what) {
     if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
-}
-
-std::string shape_str(const std::vector<int32_t> &v) {
-    std::stringstream ss;
-    for (size_t i = 0; i < v.size(); ++i) ss << (i ? "," : "") << v[i];
-    return ss.str();
-}
-
-// pads / strides arrive with 2 or 4 entries; 4 entries must be symmetric (dabnn/net.cpp:174-185)
-void check_symmetric(const std::vector<int32_t> &v, const char *what) {
-    BNN_ASSERT(v.size() == 2 || (v.size() == 4 && v[0] == v[2] && v[1] == v[3]),
-               std::string(what) + " must have 2 entries or 4 symmetric ones, got " + shape_str(v));
 }
 
 }  // namespace
@@ -107,19 +79,32 @@ void Net::read(const std::string &path) {
     f.seekg(0);
     file_.resize((size_t)size);
     if (!f.read(reinterpret_cast<char *>(file_.data()), size)) throw std::invalid_argument("Read file error " + path);
-    prepare(file_.data());
+    prepare(file_.data(), file_.size());
     file_.clear();
     file_.shrink_to_fit();
 }
 
 void Net::read_buf(const void *ptr) {
+    // the reference's signature (dabnn/net.cpp:46): the extent of the buffer is unknown, so offsets are only kept
+    // from wrapping around; callers that know the size use read_buf(ptr, len)
     BNN_ASSERT(ptr != nullptr, "read_buf: null model buffer");
-    prepare(ptr);
+    prepare(ptr, SIZE_MAX);
+}
+
+void Net::read_buf(const void *ptr, size_t len) {
+    BNN_ASSERT(ptr != nullptr, "read_buf: null model buffer");
+    prepare(ptr, len);
 }
 
 void Net::add_mat(const std::string &name, std::shared_ptr<Mat> mat) { mat_map_[name] = mat; }
 
 std::shared_ptr<Mat> Net::get_blob(const std::string &name) {
+    auto m = blob(name);
+    m->sync_to_host();
+    return m;
+}
+
+std::shared_ptr<Mat> Net::blob(const std::string &name) {
     auto it = mat_map_.find(name);
     if (it == mat_map_.end()) {
         auto gone = elided_.find(name);
@@ -130,177 +115,109 @@ std::shared_ptr<Mat> Net::get_blob(const std::string &name) {
     return it->second;
 }
 
-void Net::prepare(const void *buf) {
+void Net::prepare(const void *buf, size_t len) {
     BNN_ASSERT(!prepared_, "a Net can be read once");
     BNN_ASSERT(!(strict && !run_fconv), "fconv must be run in strict mode");
-    const fb::Table model = fb::root(buf);
-    const uint32_t version = model.scalar<uint32_t>(M_VERSION, 0);
-    BNN_ASSERT(version == kModelVersion, "The model version should be " + std::to_string(kModelVersion) + ", got " +
-                                             std::to_string(version) + " instead.");
+    // parse (bounds-checked) and check the whole model on the host before anything is allocated on the device
+    ModelDesc model = parse_model(buf, len);
+    check_model(model, run_fconv);
+    for (const auto &kv : model.shapes) shapes_[kv.first] = kv.second;
 
     // inputs: the first one only (dabnn/net.cpp:59-70)
-    BNN_ASSERT(model.vec_len(M_INPUTS) >= 1, "the model has no input");
     {
-        const fb::Table in = model.vec_table(M_INPUTS, 0);
-        const auto shape = in.vec_copy<uint32_t>(I_SHAPE);
-        BNN_ASSERT(shape.size() == 4, "input shape must be NHWC");
-        input_name_ = in.str(I_NAME);
-        shapes_[input_name_] = shape;
-        add_mat(input_name_, std::make_shared<Mat>(batch_, shape[1], shape[2], shape[3], DataType::Float, input_name_));
+        const InputDesc &in = model.inputs[0];
+        input_name_ = in.name;
+        add_mat(input_name_, std::make_shared<Mat>(batch_, in.shape[1], in.shape[2], in.shape[3], DataType::Float, input_name_));
     }
 
     // initializers (dabnn/net.cpp:72-138), uploaded to the device
-    for (uint32_t i = 0; i < model.vec_len(M_INITIALIZERS); ++i) {
-        const fb::Table t = model.vec_table(M_INITIALIZERS, i);
-        const std::string name = t.str(T_NAME);
-        const auto shape = t.vec_copy<uint32_t>(T_SHAPE);
-        shapes_[name] = shape;
-        if (t.scalar<int8_t>(T_DATA_TYPE, 0) == 1) {  // Bit
-            BNN_ASSERT(shape.size() == 4, "bit tensor " + name + " must be 4-D");
-            uint32_t len = 0;
-            const uint64_t *data = t.vec<uint64_t>(T_BIN_DATA, &len);
-            BNN_ASSERT(len > 0 && len % shape[0] == 0, "bit tensor " + name + " has a bad length");
+    for (const TensorDesc &t : model.initializers) {
+        std::shared_ptr<Mat> m;
+        if (t.is_bit) {
             // shape is [n][kh][kw][c]; the word count per filter may include the padding to 128 bits
-            auto m = std::make_shared<Mat>((size_t)len, DataType::Bit, name);
-            m->n = shape[0], m->h = shape[1], m->w = shape[2], m->c = shape[3] / 64, m->elem_c = shape[3];
-            m->upload(data, (size_t)len * 8);
-            add_mat(name, m);
+            m = std::make_shared<Mat>(t.len, DataType::Bit, t.name);
+            m->n = t.shape[0], m->h = t.shape[1], m->w = t.shape[2], m->c = t.shape[3] / 64, m->elem_c = t.shape[3];
+            m->upload(t.data, t.len * 8);
         } else {
-            uint32_t len = 0;
-            const float *data = t.vec<float>(T_FLOAT_DATA, &len);
-            size_t want = 1;
-            for (auto d : shape) want *= d;
-            BNN_ASSERT(len == want, "float tensor " + name + " does not match its shape");
-            std::shared_ptr<Mat> m;
-            if (shape.size() == 4) {
-                m = std::make_shared<Mat>((int)shape[0], (int)shape[1], (int)shape[2], (int)shape[3], DataType::Float, name);
-            } else {
-                BNN_ASSERT(shape.size() == 1, "float tensor " + name + " must be 1-D or 4-D");
-                m = std::make_shared<Mat>((size_t)shape[0], DataType::Float, name);
-            }
-            m->upload(data, (size_t)len * 4);
-            add_mat(name, m);
+            if (t.shape.size() == 4)
+                m = std::make_shared<Mat>((int)t.shape[0], (int)t.shape[1], (int)t.shape[2], (int)t.shape[3], DataType::Float, t.name);
+            else
+                m = std::make_shared<Mat>((size_t)t.shape[0], DataType::Float, t.name);
+            m->upload(t.data, t.len * 4);
         }
+        add_mat(t.name, m);
     }
 
-    auto shape_of = [&](const std::string &n) -> const std::vector<uint32_t> & {
-        auto it = shapes_.find(n);
-        if (it == shapes_.end()) throw std::out_of_range("Key " + n + " not found.");
-        return it->second;
-    };
-    auto new_output = [&](const std::string &name, uint32_t h, uint32_t w, uint32_t c) {
-        shapes_[name] = {1, h, w, c};
-        if (!has_blob(name)) add_mat(name, std::make_shared<Mat>(batch_, (int)h, (int)w, (int)c, DataType::Float, name));
+    auto new_output = [&](const std::string &name, DataType type = DataType::Float, int images = 0) {
+        const auto &s = model.shapes.at(name);
+        if (!has_blob(name))
+            add_mat(name, std::make_shared<Mat>(images ? images : batch_, (int)s[1], (int)s[2], (int)s[3], type, name));
     };
     auto alias_output = [&](const std::string &output, const std::string &input) {  // ADD_INPLACE_LAYER
-        add_mat(output, get_blob(input));
-        shapes_[output] = shape_of(input);
+        add_mat(output, blob(input));
     };
 
-    for (uint32_t i = 0; i < model.vec_len(M_LAYERS); ++i) {
-        const fb::Table layer = model.vec_table(M_LAYERS, i);
-        const int type = layer.scalar<int8_t>(L_TYPE, 0);
-        const std::string name = layer.str(L_NAME);
-        switch (type) {
-            case FpConv2D:
-            case BinConv2D: {
-                const fb::Table p = layer.table(type == FpConv2D ? L_FPCONV : L_BINCONV);
-                BNN_ASSERT(p.valid(), "conv layer without parameters");
-                const std::string input = p.str(0), weight = p.str(1), bias = p.str(2), output = p.str(6);
-                const auto pads = p.vec_copy<int32_t>(3), strides = p.vec_copy<int32_t>(4), dil = p.vec_copy<int32_t>(5);
-                check_symmetric(pads, "pads");
-                check_symmetric(strides, "strides");
-                const int dil_h = dil.size() >= 1 ? dil[0] : 1, dil_w = dil.size() >= 2 ? dil[1] : dil_h;
-                const auto &is = shape_of(input);
-                const auto &ws = shape_of(weight);  // [cout][kh][kw][cin]
-                const int pad_h = pads[0], pad_w = pads[1];
-                const uint32_t oh = (is[1] - ((ws[1] - 1) * dil_h + 1) + 2 * pad_h) / strides[0] + 1;  // common/Shaper.cpp:34-54
-                const uint32_t ow = (is[2] - ((ws[2] - 1) * dil_w + 1) + 2 * pad_w) / strides[1] + 1;
-                new_output(output, oh, ow, ws[0]);
-                if (type == BinConv2D) {
-                    BNN_ASSERT(dil_h == 1 && dil_w == 1, "BinConv dilation must be 1");
-                    layers.push_back(
-                        std::make_shared<BinConv>(get_weak(), name, input, weight, output, pad_h, pad_w, strides[0], strides[1]));
+    for (const LayerDesc &l : model.layers) {
+        switch (l.type) {
+            case kFpConv2D:
+            case kBinConv2D: {
+                new_output(l.outputs[0]);
+                if (l.type == kBinConv2D) {
+                    layers.push_back(std::make_shared<BinConv>(get_weak(), l.name, l.inputs[0], l.weight, l.outputs[0], l.pad_h,
+                                                               l.pad_w, l.stride_h, l.stride_w));
                 } else if (run_fconv) {
-                    BNN_ASSERT(dil_h == dil_w, "FloatConv needs equal dilations");
-                    if (!bias.empty())
-                        layers.push_back(std::make_shared<FloatConv>(get_weak(), name, input, weight, bias, output, pad_h,
-                                                                     pad_w, strides[0], strides[1], dil_h));
+                    if (!l.bias.empty())
+                        layers.push_back(std::make_shared<FloatConv>(get_weak(), l.name, l.inputs[0], l.weight, l.bias, l.outputs[0],
+                                                                     l.pad_h, l.pad_w, l.stride_h, l.stride_w, l.dil_h));
                     else
-                        layers.push_back(std::make_shared<FloatConv>(get_weak(), name, input, weight, output, pad_h, pad_w,
-                                                                     strides[0], strides[1], dil_h));
+                        layers.push_back(std::make_shared<FloatConv>(get_weak(), l.name, l.inputs[0], l.weight, l.outputs[0], l.pad_h,
+                                                                     l.pad_w, l.stride_h, l.stride_w, l.dil_h));
                 }
                 break;
             }
-            case AffineT: {
-                const fb::Table p = layer.table(L_AFFINE);
-                BNN_ASSERT(p.valid(), "Affine layer without parameters");
-                const std::string input = p.str(0), a = p.str(1), b = p.str(2), output = p.str(3);
-                alias_output(output, input);
-                layers.push_back(std::make_shared<Affine>(get_weak(), name, input, a, b));
+            case kAffine:
+                alias_output(l.outputs[0], l.inputs[0]);
+                layers.push_back(std::make_shared<Affine>(get_weak(), l.name, l.inputs[0], l.a, l.b));
                 break;
-            }
-            case AddT: {
-                const fb::Table p = layer.table(L_ADD);
-                BNN_ASSERT(p.valid(), "Add layer without parameters");
-                const std::string in1 = p.str(0), in2 = p.str(1), output = p.str(2);
-                alias_output(output, in1);
-                layers.push_back(std::make_shared<Add>(get_weak(), name, in1, in2));
+            case kAdd:
+                alias_output(l.outputs[0], l.inputs[0]);
+                layers.push_back(std::make_shared<Add>(get_weak(), l.name, l.inputs[0], l.inputs[1]));
                 break;
-            }
-            case ReluT: {
-                const fb::Table p = layer.table(L_RELU);
-                BNN_ASSERT(p.valid(), "Relu layer without parameters");
-                const std::string input = p.str(0), output = p.str(1);
-                alias_output(output, input);
-                layers.push_back(std::make_shared<Relu>(get_weak(), name, input));
+            case kRelu:
+                alias_output(l.outputs[0], l.inputs[0]);
+                layers.push_back(std::make_shared<Relu>(get_weak(), l.name, l.inputs[0]));
                 break;
-            }
-            case MaxPoolT:
-            case AvePoolT: {
-                const fb::Table p = layer.table(type == MaxPoolT ? L_MAXPOOL : L_AVEPOOL);
-                BNN_ASSERT(p.valid(), "pool layer without parameters");
-                const std::string input = p.str(0), output = p.str(4);
-                const auto ks = p.vec_copy<int32_t>(1), pads = p.vec_copy<int32_t>(2), strides = p.vec_copy<int32_t>(3);
-                BNN_ASSERT(ks.size() == 2 && pads.size() >= 2 && strides.size() >= 2, "pool layer with malformed attributes");
-                BNN_ASSERT(ks[0] > 0 && ks[1] > 0 && strides[0] > 0 && strides[1] > 0,
-                           "global pooling must be exported with an explicit kernel and stride");
-                const auto &is = shape_of(input);
-                const uint32_t oh = (is[1] - ks[0] + 2 * pads[0]) / strides[0] + 1;  // common/Shaper.cpp:127-145
-                const uint32_t ow = (is[2] - ks[1] + 2 * pads[1]) / strides[1] + 1;
-                new_output(output, oh, ow, is[3]);
-                if (type == MaxPoolT)
-                    layers.push_back(std::make_shared<MaxPool>(get_weak(), name, input, output, ks[0], ks[1], pads[0], pads[1],
-                                                               strides[0], strides[1]));
+            case kMaxPool:
+            case kAvePool:
+                new_output(l.outputs[0]);
+                if (l.type == kMaxPool)
+                    layers.push_back(std::make_shared<MaxPool>(get_weak(), l.name, l.inputs[0], l.outputs[0], l.kernel_shape[0],
+                                                               l.kernel_shape[1], l.pad_h, l.pad_w, l.stride_h, l.stride_w));
                 else
-                    layers.push_back(std::make_shared<AvePool>(get_weak(), name, input, output, ks[0], ks[1], pads[0], pads[1],
-                                                               strides[0], strides[1]));
+                    layers.push_back(std::make_shared<AvePool>(get_weak(), l.name, l.inputs[0], l.outputs[0], l.kernel_shape[0],
+                                                               l.kernel_shape[1], l.pad_h, l.pad_w, l.stride_h, l.stride_w));
+                break;
+            case kPRelu:
+                alias_output(l.outputs[0], l.inputs[0]);
+                layers.push_back(std::make_shared<PRelu>(get_weak(), l.name, l.inputs[0], l.slope));
+                break;
+            case kConcat:
+                new_output(l.outputs[0]);
+                layers.push_back(std::make_shared<Concat>(get_weak(), l.name, l.inputs[0], l.inputs[1], l.outputs[0]));
+                break;
+            case kSplit: {  // dabnn/net.cpp:245-250: the outputs take the input's type and image count
+                const int images = blob(l.inputs[0])->n;
+                new_output(l.outputs[0], DataType::Bit, images);
+                new_output(l.outputs[1], DataType::Bit, images);
+                layers.push_back(std::make_shared<Split>(get_weak(), l.name, l.inputs[0], l.outputs[0], l.outputs[1]));
                 break;
             }
-            case PReluT: {
-                const fb::Table p = layer.table(L_PRELU);
-                BNN_ASSERT(p.valid(), "PRelu layer without parameters");
-                const std::string input = p.str(0), slope = p.str(1), output = p.str(2);
-                alias_output(output, input);
-                layers.push_back(std::make_shared<PRelu>(get_weak(), name, input, slope));
+            case kShuffle:
+                alias_output(l.outputs[0], l.inputs[0]);
+                layers.push_back(std::make_shared<Shuffle>(get_weak(), l.name, l.inputs[0]));
                 break;
-            }
-            case ConcatT: {  // dabnn/net.cpp:230-236: two inputs, channel axis; shape as common/Shaper.cpp:157-178
-                const fb::Table p = layer.table(L_CONCAT);
-                BNN_ASSERT(p.valid(), "Concat layer without parameters");
-                BNN_ASSERT(p.scalar<int32_t>(1, 0) == 3, "Concat: axis must be 3");
-                BNN_ASSERT(p.vec_len(0) == 2, "Concat takes two inputs");
-                const std::string in1 = p.vec_str(0, 0), in2 = p.vec_str(0, 1), output = p.str(2);
-                const auto &s1 = shape_of(in1);
-                const auto &s2 = shape_of(in2);
-                BNN_ASSERT(s1[1] == s2[1] && s1[2] == s2[2], "Wrong input for concat");
-                new_output(output, s1[1], s1[2], s1[3] + s2[3]);
-                layers.push_back(std::make_shared<Concat>(get_weak(), name, in1, in2, output));
-                break;
-            }
             default:
-                throw std::runtime_error(std::string("Not supported op ") +
-                                         (type >= 0 && type <= PReluT ? kLayerTypeNames[type] : "unknown"));
+                throw std::runtime_error(std::string("Not supported op ") + layer_type_name(l.type));
         }
     }
     if (optimize) fuse_binconv_epilogues();
@@ -337,6 +254,11 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
     } else if (auto mp = std::dynamic_pointer_cast<MaxPool>(l)) {
         reads = {mp->input_mat.get()};
         writes = {mp->output_mat.get()};
+    } else if (auto sp = std::dynamic_pointer_cast<Split>(l)) {
+        reads = {sp->input_mat.get()};
+        writes = {sp->output_mat1.get(), sp->output_mat2.get()};
+    } else if (auto sh = std::dynamic_pointer_cast<Shuffle>(l)) {
+        reads = writes = {sh->data_mat.get()};
     }
 }
 
@@ -525,8 +447,8 @@ void Net::fuse_binconv_epilogues() {
 void Net::run(const void *host_input) {
     BNN_ASSERT(prepared_, "run before read");
     BNN_ASSERT(host_input != nullptr, "run: null input");
-    auto in = get_blob(input_name_);
-    hip_check(hipMemcpyAsync(in->data, host_input, in->bytes(), hipMemcpyHostToDevice, static_cast<hipStream_t>(stream_)),
+    auto in = blob(input_name_);
+    hip_check(hipMemcpyAsync(in->dev, host_input, in->bytes(), hipMemcpyHostToDevice, static_cast<hipStream_t>(stream_)),
               "hipMemcpyAsync");
     run_device(nullptr);
 }
@@ -536,8 +458,8 @@ void Net::run_device(const void *device_input) {
     BNN_ASSERT(!(strict && !run_fconv), "fconv must be run in strict mode");
     hipStream_t s = static_cast<hipStream_t>(stream_);
     if (device_input) {
-        auto in = get_blob(input_name_);
-        hip_check(hipMemcpyAsync(in->data, device_input, in->bytes(), hipMemcpyDeviceToDevice, s), "hipMemcpyAsync");
+        auto in = blob(input_name_);
+        hip_check(hipMemcpyAsync(in->dev, device_input, in->bytes(), hipMemcpyDeviceToDevice, s), "hipMemcpyAsync");
     }
     if (profile || !use_graph) {
         for (const auto &layer : layers) layer->forward();
@@ -565,6 +487,7 @@ void Net::run_device(const void *device_input) {
     }
     ++runs_;
     hip_check(hipStreamSynchronize(s), "hipStreamSynchronize");
+    for (const auto &kv : mat_map_) kv.second->mark_device_written();  // host mirrors show the previous run
 }
 
 std::vector<std::string> Net::layer_descriptions() const {

@@ -19,7 +19,7 @@
 
 namespace bnn {
 
-class Net : public std::enable_shared_from_this<Net> {
+class BNN_API Net : public std::enable_shared_from_this<Net> {
    public:
     static std::shared_ptr<Net> create();
     ~Net();
@@ -29,9 +29,14 @@ class Net : public std::enable_shared_from_this<Net> {
     const std::string &input_name() const { return input_name_; }
     void read(const std::string &path);
     void read_buf(const void *ptr);
+    void read_buf(const void *ptr, size_t len);  // the same, with every offset of the model checked against len
     void run(const void *host_input);
     void run_device(const void *device_input);
+    // The blob with its host mirror up to date (dabnn/net.cpp:288-290): `data`, operator[] ... read what the last
+    // run left on the device.
     std::shared_ptr<Mat> get_blob(const std::string &name);
+    // The same blob without the device-to-host copy (what the layers and the C ABI use).
+    std::shared_ptr<Mat> blob(const std::string &name);
     bool has_blob(const std::string &name) const { return mat_map_.count(name) != 0; }
     std::vector<std::string> layer_descriptions() const;
 
@@ -60,7 +65,7 @@ class Net : public std::enable_shared_from_this<Net> {
 
    private:
     Net();
-    void prepare(const void *model_buf);
+    void prepare(const void *model_buf, size_t len);
     void fuse_binconv_epilogues();
     std::weak_ptr<Net> get_weak() { return shared_from_this(); }
     std::vector<std::shared_ptr<Layer>> layers;

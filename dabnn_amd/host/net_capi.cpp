@@ -6,6 +6,7 @@
 #include <string>
 #include <vector>
 
+#include "model.h"
 #include "net.h"
 
 struct dabnet {
@@ -93,7 +94,15 @@ int dabnet_read_file(dabnet_t *net, const char *path) {
 int dabnet_read_buf(dabnet_t *net, const void *buf, size_t len) {
     return guarded([&] {
         if (!buf || len < 8) throw std::invalid_argument("model buffer too small");
-        net->net->read_buf(buf);
+        net->net->read_buf(buf, len);
+    });
+}
+
+int dabnet_check_model(const void *buf, size_t len, int run_fconv) {
+    return guarded([&] {
+        if (!buf || len < 8) throw std::invalid_argument("model buffer too small");
+        bnn::ModelDesc model = bnn::parse_model(buf, len);
+        bnn::check_model(model, run_fconv != 0);
     });
 }
 
@@ -112,7 +121,7 @@ const char *dabnet_input_name(dabnet_t *net) { return net->net->input_name().c_s
 
 int dabnet_blob_info(dabnet_t *net, const char *name, int shape[4], int *is_bit, size_t *bytes) {
     return guarded([&] {
-        auto m = net->net->get_blob(name ? name : "");
+        auto m = net->net->blob(name ? name : "");
         if (shape) shape[0] = m->n, shape[1] = m->h, shape[2] = m->w, shape[3] = m->c;
         if (is_bit) *is_bit = m->data_type == bnn::DataType::Bit;
         if (bytes) *bytes = m->bytes();
@@ -121,7 +130,7 @@ int dabnet_blob_info(dabnet_t *net, const char *name, int shape[4], int *is_bit,
 
 int dabnet_get_blob(dabnet_t *net, const char *name, void *host_out, size_t bytes) {
     return guarded([&] {
-        auto m = net->net->get_blob(name ? name : "");
+        auto m = net->net->blob(name ? name : "");
         if (!host_out) throw std::runtime_error("get_blob: null destination");
         m->download(host_out, bytes);
     });

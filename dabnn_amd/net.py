@@ -35,6 +35,7 @@ NET_SIGNATURES = {
     "dabnet_time_report": (_cp, [_vp]),
     "dabnet_read_file": (_i, [_vp, _cp]),
     "dabnet_read_buf": (_i, [_vp, _vp, _sz]),
+    "dabnet_check_model": (_i, [_vp, _sz, _i]),
     "dabnet_run": (_i, [_vp, _vp]),
     "dabnet_run_device": (_i, [_vp, _vp]),
     "dabnet_input_name": (_cp, [_vp]),
@@ -58,6 +59,12 @@ def _check(rc):
     if rc == DABNET_EKEY:
         raise KeyError(msg)  # StrKeyMap::at
     raise RuntimeError(msg)  # std::runtime_error
+
+
+def check_model(buf, run_fconv=True):
+    """Parse and check a .dab model on the host (no GPU): raises what Net.read_buf would raise for it."""
+    b = bytes(buf)
+    _check(hostlib.dabnet_check_model(b, len(b), int(run_fconv)))
 
 
 class Net:

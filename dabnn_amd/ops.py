@@ -73,6 +73,24 @@ def pad(x, pad_h, pad_w):
     return out
 
 
+def split_bit(x):
+    """Split::forward_impl (dabnn/layers/Split.cpp:6-21): packed [..., CW] -> two packed [..., CW/2]."""
+    _need(x, torch.int64, "x")
+    cw = x.shape[-1]
+    half = tuple(x.shape[:-1]) + (max(cw // 2, 1),)
+    o1, o2 = _empty(half, torch.int64, x.device), _empty(half, torch.int64, x.device)
+    check(lib.dab_split_bit(_ptr(x), x.numel() // max(cw, 1), cw, _ptr(o1), _ptr(o2), _stream()))
+    return o1, o2
+
+
+def shuffle_bit_inplace(x):
+    """Shuffle::forward_impl (dabnn/layers/Shuffle.cpp:6-43), in place on packed [..., CW]."""
+    _need(x, torch.int64, "x")
+    cw = x.shape[-1]
+    check(lib.dab_shuffle_bit_inplace(_ptr(x), x.numel() // max(cw, 1), cw * 64, _stream()))
+    return x
+
+
 def fused_binarize_im2col(x, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h=1, dil_w=1):
     """fused_binarize_im2col (dabnn/fused_binarize_im2col.h:6-68): -> int64 [N*OH*OW, row_words]."""
     _need(x, torch.float32, "x")

@@ -72,6 +72,21 @@ DAB_API int dab_pad_bit(const uint64_t *x, int n, int h, int w, int cw, int pad_
                 dab_stream_t stream);
 
 /*
+ * Split::forward_impl (dabnn/layers/Split.cpp:6-21) on packed activations: the cw words of each of the n_pix pixels
+ * are cut in two, out1 takes words [0, cw/2), out2 words [cw/2, cw); both hold n_pix * cw/2 words.  cw * 64 channels
+ * must be a multiple of 128 and at most 512 (dabnn/layers/Split.h:22-23), i.e. cw in {2, 4, 6, 8}.
+ */
+DAB_API int dab_split_bit(const uint64_t *x, int64_t n_pix, int cw, uint64_t *out1, uint64_t *out2, dab_stream_t stream);
+
+/*
+ * Shuffle::forward_impl (dabnn/layers/Shuffle.cpp:6-43), in place on packed activations of elem_c channels
+ * (a multiple of 128, at most 512, dabnn/layers/Shuffle.h:19-20): the channel shuffle of a two-group network at the
+ * granularity the reference has -- 128 channels: the 32-bit quarters 1 and 2 of every pixel change places; 256: words
+ * 1 and 2; 512: words 2,3 and 4,5; 384 channels pass unchanged, as in the reference.
+ */
+DAB_API int dab_shuffle_bit_inplace(uint64_t *x, int64_t n_pix, int elem_c, dab_stream_t stream);
+
+/*
  * fused_binarize_im2col (dabnn/fused_binarize_im2col.h:6-68): for every
  * output pixel gather kh*kw runs of c floats (zeros outside the image),
  * zero-extend to a multiple of 128 floats and sign-pack.

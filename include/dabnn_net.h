@@ -54,6 +54,16 @@ DABNET_API const char *dabnet_time_report(dabnet_t *net);
 DABNET_API int dabnet_read_file(dabnet_t *net, const char *path);
 DABNET_API int dabnet_read_buf(dabnet_t *net, const void *buf, size_t len);
 
+/*
+ * No counterpart in the reference, which trusts the file: parses the model with every FlatBuffers offset checked against
+ * len and runs the checks of Net::prepare (dabnn/net.cpp:56-270: version, shapes as common/Shaper.cpp, symmetric pads,
+ * supported layer types, tensor sizes against layer geometry) on the host only -- no GPU is touched, nothing is built.
+ * DABNET_OK, DABNET_EINVALID (truncated or corrupt buffer), DABNET_ERUNTIME (a BNN_ASSERT of the reference, or a tensor
+ * that does not fit its layer) or DABNET_EKEY (a layer names a blob that does not exist).  dabnet_read_buf and
+ * dabnet_read_file run the same checks before they allocate.
+ */
+DABNET_API int dabnet_check_model(const void *buf, size_t len, int run_fconv);
+
 /* Net::run (dabnn/net.cpp:272-286): host_input holds batch x H x W x C floats (NHWC). Blocks until done. */
 DABNET_API int dabnet_run(dabnet_t *net, const float *host_input);
 /* Same with the input already in device memory. */

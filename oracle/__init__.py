@@ -83,6 +83,10 @@ def lib():
         L.orc_prelu_inplace.argtypes = [fp, sz, i, fp, i]
         L.orc_concat.restype = None
         L.orc_concat.argtypes = [fp, i, fp, i, sz, fp]
+        L.orc_split_bit.restype = None
+        L.orc_split_bit.argtypes = [up, sz, i, up, up]
+        L.orc_shuffle_bit.restype = None
+        L.orc_shuffle_bit.argtypes = [up, sz, i]
         L.orc_ave_pool.restype = None
         L.orc_ave_pool.argtypes = [fp, i, i, i, i, i, i, i, i, i, fp]
         L.orc_max_pool.restype = None
@@ -322,6 +326,29 @@ def concat(a, b):
     out = np.empty(a.shape[:-1] + (ca + cb,), dtype=np.float32)
     lib().orc_concat(ap, ca, bp, cb, a.size // ca, out.ctypes.data_as(_c_float_p))
     return out
+
+
+def split_bit(x):
+    """dabnn/layers/Split.cpp:6-21: packed [..., cw] -> two packed [..., cw/2]; the channel count must be a multiple
+    of 128 and at most 512 (dabnn/layers/Split.h:22-23)."""
+    x, xp = _u(x)
+    cw = x.shape[-1]
+    if (cw * 64) % 128 != 0 or cw * 64 > 512:
+        raise RuntimeError("Split: %d channels" % (cw * 64))
+    o1 = np.empty(x.shape[:-1] + (cw // 2,), dtype=np.uint64)
+    o2 = np.empty_like(o1)
+    lib().orc_split_bit(xp, x.size // cw, cw, o1.ctypes.data_as(_c_u64_p), o2.ctypes.data_as(_c_u64_p))
+    return o1, o2
+
+
+def shuffle_bit(x):
+    """dabnn/layers/Shuffle.cpp:6-43 in place on packed [..., cw] (uint64, contiguous)."""
+    assert x.dtype == np.uint64 and x.flags["C_CONTIGUOUS"]
+    cw = x.shape[-1]
+    if (cw * 64) % 128 != 0 or cw * 64 > 512:
+        raise RuntimeError("Shuffle: %d channels" % (cw * 64))  # dabnn/layers/Shuffle.h:19-20
+    lib().orc_shuffle_bit(x.ctypes.data_as(_c_u64_p), x.size // cw, cw * 64)
+    return x
 
 
 def ave_pool(x, kh, kw, pad_h, pad_w, stride_h, stride_w):

@@ -33,6 +33,9 @@
  *   orc_prelu_inplace              torch.nn.functional.prelu (scalar and per-
  *                                  channel slope)
  *   orc_concat                     numpy.concatenate along the channel axis
+ *   orc_split_bit                  numpy slicing of the word axis
+ *   orc_shuffle_bit                a channel permutation of the unpacked bits:
+ *                                  two groups, 32 / 64 / 128 channels a piece
  *   orc_pack_weight / orc_bn_fold  K - 2*cnt end-to-end identity
  */
 #include <stddef.h>
@@ -451,6 +454,56 @@ ORC_API void orc_concat(const float *a, int ca, const float *b, int cb, size_t n
         out += ca;
         memcpy(out, b + p * cb, (size_t)cb * sizeof(float));
         out += cb;
+    }
+}
+
+/*
+ * dabnn/layers/Split.cpp:6-21: per pixel, the first c/2 words go to out1, the
+ * other c/2 to out2 (c = words per pixel).
+ */
+ORC_API void orc_split_bit(const uint64_t *x, size_t n_pix, int c, uint64_t *out1, uint64_t *out2) {
+    const int c_per_output = c / 2;
+    for (size_t p = 0; p < n_pix; ++p) {
+        memcpy(out1, x, (size_t)c_per_output * sizeof(uint64_t));
+        out1 += c_per_output;
+        x += c_per_output;
+        memcpy(out2, x, (size_t)c_per_output * sizeof(uint64_t));
+        out2 += c_per_output;
+        x += c_per_output;
+    }
+}
+
+/*
+ * dabnn/layers/Shuffle.cpp:6-43, in place: 128 channels -- 32-bit quarters 1
+ * and 2 of a pixel change places; 256 -- words 1 and 2; 512 -- words 2,3 and
+ * 4,5; other channel counts are left alone (the reference has no branch for
+ * them).  n_pix pixels of elem_c / 64 words.
+ */
+ORC_API void orc_shuffle_bit(uint64_t *x, size_t n_pix, int elem_c) {
+    if (elem_c == 128) {
+        uint32_t *ptr = (uint32_t *)x;
+        for (size_t p = 0; p < n_pix; ++p) {
+            const uint32_t tmp = ptr[1];
+            ptr[1] = ptr[2];
+            ptr[2] = tmp;
+            ptr += 4;
+        }
+    } else if (elem_c == 256) {
+        for (size_t p = 0; p < n_pix; ++p) {
+            const uint64_t tmp = x[1];
+            x[1] = x[2];
+            x[2] = tmp;
+            x += 4;
+        }
+    } else if (elem_c == 512) {
+        for (size_t p = 0; p < n_pix; ++p) {
+            const uint64_t tmp1 = x[2], tmp2 = x[3];
+            x[2] = x[4];
+            x[3] = x[5];
+            x[4] = tmp1;
+            x[5] = tmp2;
+            x += 8;
+        }
     }
 }
 

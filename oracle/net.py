@@ -62,6 +62,15 @@ def _apply(layer, act, blobs, record=None):
         fn = orc.max_pool if ty == "MaxPool" else orc.ave_pool
         act[layer["output"]] = fn(src, kh, kw, layer["pads"][0], layer["pads"][1], layer["strides"][0],
                                   layer["strides"][1])
+    elif ty == "Split":  # dabnn/net.cpp:245-250
+        o1, o2 = orc.split_bit(act[layer["input"]])
+        act[layer["outputs"][0]], act[layer["outputs"][1]] = o1, o2
+    elif ty == "Shuffle":  # dabnn/net.cpp:251-256, in place
+        buf = act[layer["input"]]
+        if buf.dtype != np.uint64:
+            raise RuntimeError("Shuffle only supports bit mat")
+        orc.shuffle_bit(buf)
+        act[layer["output"]] = buf
     else:
         raise RuntimeError("Not supported op " + ty)
 

@@ -84,6 +84,26 @@ def test_pad_bit(dab, n, h, w, cw, ph, pw):
     np.testing.assert_array_equal(got, want)
 
 
+# ---------------------------------------------------------------- Split / Shuffle on packed words
+@pytest.mark.parametrize("shape", [(1, 4, 6, 2), (3, 7, 7, 4), (2, 5, 3, 6), (5, 14, 14, 8), (64, 28, 28, 4)])
+def test_split_and_shuffle_bit(dab, shape):
+    x = rng(5).integers(0, 2**64, size=shape, dtype=np.uint64)
+    o1, o2 = dab.split_bit(dev_u(x))
+    w1, w2 = orc.split_bit(x)
+    np.testing.assert_array_equal(host_u(o1), w1)
+    np.testing.assert_array_equal(host_u(o2), w2)
+    np.testing.assert_array_equal(host_u(dab.shuffle_bit_inplace(dev_u(x))), orc.shuffle_bit(x.copy()))
+
+
+def test_split_and_shuffle_reject_other_channel_counts(dab):
+    for cw in (1, 3, 10):
+        x = torch.zeros((1, 2, 2, cw), dtype=torch.int64, device="cuda")
+        with pytest.raises(RuntimeError, match="Split: %d channels" % (cw * 64)):
+            dab.split_bit(x)
+        with pytest.raises(RuntimeError, match="Shuffle: %d channels" % (cw * 64)):
+            dab.shuffle_bit_inplace(x)
+
+
 # ---------------------------------------------------------------- fused_binarize_im2col
 @pytest.mark.parametrize("n,h,w,c,k,pad,stride,dil", [
     (1, 8, 8, 128, 3, 1, 1, 1), (2, 8, 8, 64, 3, 1, 2, 1), (1, 7, 9, 192, 3, 1, 1, 1), (1, 6, 6, 128, 5, 2, 2, 1),

@@ -331,13 +331,94 @@ def test_error_paths(mods, tmp_path):
     with pytest.raises(RuntimeError, match="Not supported op Softmax"):
         net.Net().read_buf(df.write_model(bad, inits, inputs))
     shuffle = [{"type": "Shuffle", "name": "sh", "input": "data", "output": "out"}]
-    with pytest.raises(RuntimeError, match="Not supported op Shuffle"):
+    with pytest.raises(RuntimeError, match="Shuffle only supports bit mat"):  # dabnn/layers/Shuffle.h:16-18
         net.Net().read_buf(df.write_model(shuffle, [], [("data", [1, 4, 4, 128])]))
+    # a weight tensor shorter than the layer's geometry is refused before any kernel could read past it
+    wp = models.pack_weight(np.ones((8, 3, 3, 128), np.float32))
+    short = [{"name": "w", "shape": [8, 3, 3, 128], "data": np.ascontiguousarray(wp[:, :16]).ravel(), "align_hwc_to_128": True}]
+    conv = [{"type": "BinConv2D", "name": "bc", "input": "data", "weight": "w", "output": "cnt", "pads": [1] * 4,
+             "strides": [1, 1], "dilations": [1, 1]}]
+    with pytest.raises(RuntimeError, match="words per filter"):
+        net.Net().read_buf(df.write_model(conv, short, [("data", [1, 8, 8, 128])]))
+    good = df.write_model(layers, inits, inputs)
+    with pytest.raises(ValueError, match="malformed model buffer"):  # std::invalid_argument
+        net.Net().read_buf(good[:len(good) // 2])
     n = net.Net().read_buf(df.write_model(layers, inits, inputs))
     with pytest.raises(KeyError):
         n.get_blob("no_such_blob")
     with pytest.raises(ValueError):
         n.run(np.zeros((1, 8, 8, 3), dtype=np.float32))
+    n.close()
+
+
+def test_split_and_shuffle_layers_on_bit_blobs(mods):
+    """dabnn/net.cpp:245-256: Shuffle works in place on a Bit blob, Split cuts it into two Bit blobs.  No layer of
+    the reference's Net produces a Bit blob, so the input is a Bit initializer, as in the reference."""
+    df, models, net = mods
+    r = np.random.default_rng(15)
+    for c in (128, 256, 384, 512):
+        words = r.integers(0, 2**64, size=(3, 5, 4, c // 64), dtype=np.uint64)
+        inits = [{"name": "bits", "shape": [3, 5, 4, c], "data": words.ravel(), "align_hwc_to_128": False}]
+        layers = [{"type": "Shuffle", "name": "sh", "input": "bits", "output": "shuffled"},
+                  {"type": "Split", "name": "sp", "input": "shuffled", "outputs": ["left", "right"]}]
+        n = net.Net(batch=2).read_buf(df.write_model(layers, inits, [("data", [1, 4, 4, 64])]))
+        assert [d.split()[0] for d in n.layers()] == ["Shuffle", "Split"]
+        n.run(np.zeros((2, 4, 4, 64), np.float32))
+        want = orc.shuffle_bit(words.copy())
+        l, rgt = orc.split_bit(want)
+        np.testing.assert_array_equal(n.get_blob("shuffled").reshape(want.shape), want)
+        np.testing.assert_array_equal(n.get_blob("bits").reshape(want.shape), want)  # in place: the names alias
+        np.testing.assert_array_equal(n.get_blob("left").reshape(l.shape), l)
+        np.testing.assert_array_equal(n.get_blob("right").reshape(rgt.shape), rgt)
+        n.close()
+
+
+def test_flatc_style_encoding_loads(mods):
+    """Files written the way flatc's builders write them -- default scalars left out (Float32 tensors, the FpConv2D
+    layer type, align_hwc_to_128 = false), equal vtables shared, trailing absent slots trimmed from every vtable,
+    four-entry symmetric pads -- give the same network as the untrimmed encoding."""
+    df, models, net = mods
+    layers, inits, inputs = models.small_bnn(5, hw=16, width=64)
+    assert any(len(l.get("pads", [])) == 4 for l in layers)
+    plain = df.write_model(layers, inits, inputs)
+    trimmed = df.write_model(layers, inits, inputs, trim_vtables=True)
+    assert len(trimmed) < len(plain)
+    x = np.random.default_rng(16).standard_normal((2, 16, 16, 3)).astype(np.float32)
+    outs = []
+    for buf in (plain, trimmed):
+        n = net.Net(batch=2).read_buf(buf)
+        outs.append(n.layers())
+        n.run(x)
+        outs.append(n.get_blob("logits").copy())
+        n.close()
+    assert outs[0] == outs[2]
+    np.testing.assert_array_equal(outs[1], outs[3])
+
+
+def test_cpp_callers_of_the_reference_work_unchanged(mods, tmp_path):
+    """tests/cpp/net_api_test.cpp is the reference's own usage (tests/net_test.cpp:29-50,63-65, JavaWrapper.cpp:56-60,
+    binaries/run.cpp:41-50) compiled against this library's C++ headers: optimize = false and optimize = true agree
+    through Mat::operator==, and get_blob hands back host-readable data through data, operator T*, operator[]."""
+    import os
+    import subprocess
+    df, models, net = mods
+    exe = os.path.join(os.path.dirname(os.path.abspath(net.__file__)), "lib", "net_api_test")
+    assert os.path.exists(exe), "build it with make -C dabnn_amd/host"
+    layers, inits, inputs = models.small_bnn(6, hw=16, width=64)
+    path = tmp_path / "small.dab"
+    path.write_bytes(df.write_model(layers, inits, inputs))
+    out = subprocess.run([exe, str(path), "logits", str(16 * 16 * 3), "binaized_for_b0_cnt_cal"], capture_output=True,
+                         text=True, timeout=120)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.strip().endswith("ok")
+    n = net.Net(batch=1).read_buf(path.read_bytes())
+    n.run(np.ones((1, 16, 16, 3), np.float32))
+    want = n.get_blob("logits").ravel()
+    got = [float(l.split()[2]) for l in out.stdout.splitlines() if l.startswith("v ")]
+    assert len(got) == 8
+    np.testing.assert_array_equal(np.array(got, np.float32), want[:8])
+    w0 = [int(l.split()[1]) for l in out.stdout.splitlines() if l.startswith("w0 ")]
+    assert w0 == [int(n.get_blob("binaized_for_b0_cnt_cal").ravel()[0])]
     n.close()
 
 

@@ -411,3 +411,55 @@ def test_run_segments_fed_with_its_own_blobs_reproduces_the_layer_loop():
             np.testing.assert_array_equal(want, cpu[name])
             count += 1
         assert count == (7 if hw == 16 else 28)
+
+
+# ---------------------------------------------------------------- Split / Shuffle on packed words
+def _unpack_bits(words, c):
+    """uint64 [..., cw] -> uint8 bits [..., c], bit j of word i = channel 64*i + j."""
+    b = np.unpackbits(words[..., None].view(np.uint8), axis=-1, bitorder="little")
+    return b.reshape(words.shape[:-1] + (c,))
+
+
+@pytest.mark.parametrize("c", [128, 256, 384, 512])
+def test_split_bit_is_a_slice_of_the_channel_axis(c):
+    """dabnn/layers/Split.cpp:6-21: output 1 holds channels [0, c/2), output 2 channels [c/2, c), checked on the
+    unpacked bits (numpy slicing), so that a mixed-up half or word order fails."""
+    r = np.random.default_rng(60)
+    x = r.integers(0, 2**64, size=(3, 5, c // 64), dtype=np.uint64)
+    o1, o2 = orc.split_bit(x)
+    bits = _unpack_bits(x, c)
+    np.testing.assert_array_equal(_unpack_bits(o1, c // 2), bits[..., :c // 2])
+    np.testing.assert_array_equal(_unpack_bits(o2, c // 2), bits[..., c // 2:])
+
+
+def test_split_bit_rejects_other_channel_counts():
+    for cw in (1, 3, 10):
+        with pytest.raises(RuntimeError, match="Split"):
+            orc.split_bit(np.zeros((2, 2, cw), dtype=np.uint64))
+
+
+@pytest.mark.parametrize("c,group", [(128, 32), (256, 64), (512, 128)])
+def test_shuffle_bit_is_a_channel_permutation(c, group):
+    """dabnn/layers/Shuffle.cpp:6-43 read as a permutation of channels: the channels form four runs of `group`
+    (a b c d) and come out as a c b d -- the two-group channel shuffle at that granularity; applying it twice
+    is the identity."""
+    r = np.random.default_rng(61)
+    x = r.integers(0, 2**64, size=(4, 3, c // 64), dtype=np.uint64)
+    bits = _unpack_bits(x, c)
+    y = orc.shuffle_bit(x.copy())
+    if c == 512:
+        # the reference swaps words 2,3 with words 4,5 of the eight: runs of 128 channels, 1 and 2 change places
+        want = np.concatenate([bits[..., :128], bits[..., 256:384], bits[..., 128:256], bits[..., 384:]], axis=-1)
+    else:
+        q = bits.reshape(bits.shape[:-1] + (4, group))
+        want = q[..., [0, 2, 1, 3], :].reshape(bits.shape)
+    np.testing.assert_array_equal(_unpack_bits(y, c), want)
+    np.testing.assert_array_equal(orc.shuffle_bit(y.copy()), x)
+
+
+def test_shuffle_bit_leaves_384_channels_alone_and_rejects_the_rest():
+    x = np.random.default_rng(62).integers(0, 2**64, size=(2, 2, 6), dtype=np.uint64)
+    np.testing.assert_array_equal(orc.shuffle_bit(x.copy()), x)  # no branch for 384 in the reference
+    for cw in (1, 3, 10):
+        with pytest.raises(RuntimeError, match="Shuffle"):
+            orc.shuffle_bit(np.zeros((1, 1, cw), dtype=np.uint64))
