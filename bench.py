@@ -52,9 +52,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-side CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample")
-    ap.add_argument("--profile-mode", action="store_true",
-                    help="for rocprofv3 runs: only the headline workload (same graph replay as the timed region), preceded "
-                         "by one 256 MiB device-to-device copy that calibrates the FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--profile-mode", nargs="?", const="headline", default=None, choices=["headline", "fconv", "bireal18"],
+                    help="for rocprofv3 runs, one workload only, preceded by one 256 MiB device-to-device copy that "
+                         "calibrates the FETCH_SIZE / WRITE_SIZE counters.  headline (default): the same graph replay as "
+                         "the timed region; fconv: the float convolutions of the Bi-Real-18 stems at batch 256, three "
+                         "launches each, the two a MaxPool follows also as the one-pass kernel; bireal18: --steps runs "
+                         "of Bi-Real-18 (7x7 stem) at batch 256 through the C++ Net, layer by layer (no graph)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no exchange between images, run it with --gpus 1 "
@@ -112,6 +115,47 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)  # 256 MiB read + 256 MiB written
         torch.cuda.synchronize()
+        del src, dst
+    if args.profile_mode == "fconv":
+        shapes = [  # n, h = w, c, cout, k, pad, stride
+            (256, 224, 3, 64, 7, 3, 2), (256, 224, 3, 32, 3, 1, 2), (256, 112, 32, 32, 3, 1, 1), (256, 112, 32, 64, 3, 1, 1),
+            (256, 28, 64, 128, 1, 0, 1), (256, 1, 512, 1000, 1, 0, 1)]
+        launched = []
+        for (n, h, c, cout, k, pad, stride) in shapes:
+            x = torch.randn((n, h, h, c), generator=g).cuda()
+            w = torch.randn((cout, k, k, c), generator=g).cuda()
+            a, b = torch.randn(cout, generator=g).cuda(), torch.randn(cout, generator=g).cuda()
+            for _ in range(3):
+                dab.fconv_affine_relu(x, w, None, a, b, True, k, k, pad, pad, stride, stride)
+            torch.cuda.synchronize()
+            launched.append("%dx%dx%dx%d -> %d, %dx%d stride %d" % (n, h, h, c, cout, k, k, stride))
+            if (h + 2 * pad - k) // stride + 1 == 112 and cout == 64:
+                # the last convolution of a stem with its MaxPool 3x3 stride 2 in one pass
+                for _ in range(3):
+                    dab.fconv_maxpool(x, w, None, a, b, True, k, k, pad, pad, stride, stride, want_sign=True)
+                torch.cuda.synchronize()
+                launched.append("  the same + MaxPool 3x3 stride 2 + sign bits, one pass")
+        print(json.dumps({"profile_mode": "fconv", "launched_3x_each": launched}))
+        return
+    if args.profile_mode == "bireal18":
+        from dabnn_amd import dab_format, models
+        from dabnn_amd import net as dabnet
+        mlayers, minits, minputs = models.bireal18(2024, stem=False)
+        net = dabnet.Net(batch=256).read_buf(dab_format.write_model(mlayers, minits, minputs))
+        net.set_use_graph(False)  # every layer a dispatch of its own, in layer order
+        x = torch.randn((256, 224, 224, 3), generator=g).cuda()
+        for _ in range(max(1, args.warmup)):
+            net.run(x)
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < 0.04:
+            net.run(x)
+        for _ in range(args.steps):
+            net.run(x)
+        print(json.dumps({"profile_mode": "bireal18", "batch": 256, "runs_after_warmup": args.steps,
+                          "layers": net.layers()}))
+        net.close()
+        return
+    if args.profile_mode:
         step()
         torch.cuda.synchronize()
         pgraph = torch.cuda.CUDAGraph()

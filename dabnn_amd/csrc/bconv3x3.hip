@@ -77,6 +77,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     constexpr int WCH = Residency<CW, NARROW>::window;
     constexpr int WU = WCH / Q;  // units per staging window
     constexpr int kStageBytes = Stage<WCH>::bytes;
+    constexpr bool kPrefetchFilters = true;
     constexpr int kFlushGroup = CW == 1 ? 8 : CW == 2 ? (NARROW ? 8 : 2) : CW == 4 ? 4 : 1;  // shortcut loads in flight, as the register budget allows
     __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWavesPerBlock * kStageBytes];
     const int lane = threadIdx.x & 63;
@@ -89,21 +90,23 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     if (i0 >= i1) return;
     const int u0 = i0 * S, u1 = i1 * S;
 
-    if constexpr (CW == 8) {
-        // The filters of 512 input channels are 295 KB and more that every wave walks through with scalar loads.
-        // When other kernels have run in between they are in no L2 any more, and the first wave to need a row waits
-        // for memory in the middle of its unit.  So the launch first touches every 128-byte line of the filters once
-        // per XCD (blocks are dealt to the eight XCDs in turn: block b runs on XCD b % 8): wave j of an XCD asks for
-        // one dword of each of the lines 64*j .. 64*j+63, straight into an LDS scratch line that nobody reads, with
-        // no register and no wait involved.
-        __shared__ uint32_t prefetch_dump[kWavesPerBlock * 64];
-        const uint32_t n_lines = (uint32_t)(p.cout * 9 * CW * 8) >> 7;
+    if constexpr (kPrefetchFilters) {
+        // Every wave walks the filters with scalar loads.  When other kernels have run in between they are in no L2
+        // any more, and the first wave of an XCD to need a row waits for memory in the middle of its unit.  So the
+        // launch first touches every 128-byte line of the filters once per XCD (blocks are dealt to the eight XCDs in
+        // turn: block b runs on XCD b % 8): wave j of an XCD asks for one dword of each of the lines 64*j .. 64*j+63,
+        // straight into the first 256 bytes of its own staging buffer, with no register and no wait involved; the
+        // wave waits for it before it stages its first results there (by then the loads are long done: they were
+        // issued before the activations the first unit has just used).
+        const uint32_t n_lines = ((uint32_t)(p.cout * 9 * CW * 8) + 127u) >> 7;
         const uint32_t first = (uint32_t)((blockIdx.x >> 3) * kWavesPerBlock + wib) * 64u;
         if (first < n_lines) {
             const uint32_t line = first + lane < n_lines ? first + lane : n_lines - 1;
+            const uint32_t last_byte = (uint32_t)(p.cout * 9 * CW * 8) - 4u;
+            const uint32_t byte = line * 128u < last_byte ? line * 128u : last_byte;
             __builtin_amdgcn_global_load_lds(
-                (const void __attribute__((address_space(1))) *)(reinterpret_cast<const unsigned char *>(p.w) + (size_t)line * 128),
-                (void __attribute__((address_space(3))) *)(prefetch_dump + wib * 64), 4, 0, 0);
+                (const void __attribute__((address_space(1))) *)(reinterpret_cast<const unsigned char *>(p.w) + byte),
+                (void __attribute__((address_space(3))) *)stage, 4, 0, 0);
         }
     }
     const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
@@ -180,8 +183,17 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             __builtin_amdgcn_s_setprio(0);
         }
         uint32_t acc[Q];
-        unit_rowmajor<K32, Q, (CW >= 2 ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
+        // One vector of filters per wait: the launch has put the filters into its XCD's L2 (above), so a scalar-cache
+        // miss is short, and the second vector's 32 SGPRs are worth more elsewhere (seven batch-64 shapes in a step:
+        // 95.7 us against 98.8 with two vectors per wait, 117 with one vector and filters that start cold).  With an
+        // epilogue and 256 or 512 input channels the memory pipes are busy with the shortcut and the filters are
+        // large: there two vectors per wait win at batch 256 (51 against 59 us, 54 against 55; 0.4-0.7 us lost at
+        // batch 64).
+        unit_rowmajor<K32, Q, ((MODE != kModeCounts && CW >= 4) ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
         const int slot = cg % WU;
+        if constexpr (kPrefetchFilters) {
+            if (u == u0) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the filter prefetch wrote into the staging buffer
+        }
         stage_put<WCH, Q>(stage, lane, slot * Q, acc);
 
         // The window goes out when it is full or the tile ends.  The last unit of the wave leaves the loop first:
@@ -202,8 +214,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             ++cg;
         }
     }
-    // the filter prefetch wrote into this block's LDS: it has long arrived, but no wave leaves before that is certain
-    if constexpr (CW == 8) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 

@@ -103,9 +103,14 @@ constexpr int kMaxCount = (1 << 23) - 1;
 // the reference's weight layout): Q*K32 dwords read as vectors of 16 (or 8).
 // BV = vectors per wait.  A wait can only be "all outstanding scalar loads",
 // so the latency cover of a batch is the vector work of the previous one: one
-// vector (32 vector instructions) covers a scalar-cache hit, two ride out a
-// miss to L2 (operands too large for the 16 KiB scalar cache).
+// vector (32 vector instructions, times the other waves of the SIMD) covers a
+// scalar-cache miss that hits the L2; two ride out a miss to memory, at the
+// price of 32 more SGPRs.
 // acc is an output: acc[q] = 2^23 pattern + mismatch count of channel q.
+// (Tried and dropped: loading the first batch of a wave's next unit behind the last batch of the current one, so
+// that no unit starts with a wait.  7.07 -> 6.88 cycles per pair for the bare unit body at four waves per SIMD, but
+// in the kernel the 16-32 SGPRs that then live across the store pass cost more than the wait: 97.9 against 95.7 us
+// for the seven batch-64 shapes.)
 template <int K32, int Q, int BV_WANTED = 1>
 __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[Q]) {
     constexpr int D = Q * K32;
