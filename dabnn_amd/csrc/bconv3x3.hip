@@ -37,10 +37,15 @@ struct BconvArgs {
 
 constexpr int kWavesPerBlock = 4;
 
-// Channels per unit for CW words per pixel: units stay near 600 VALU instructions.
-template <int CW>
+// Channels per unit for CW words per pixel: units stay near 600 VALU instructions, so that the tail of a launch (one
+// unit on a lone wave) stays short and the SIMDs' loads differ by little.  256 and 512 input channels have a second
+// build with units twice that size for problems large enough that neither matters (BIG: eight channels for 256,
+// four for 512): a unit starts with a wait for its first vector of filters that only other waves can hide and ends
+// with a staging write, and half as many of both are worth 2.5 % (256 channels) and 11 % (512) at batch 256, against
+// a loss of 3-8 % at batch 64.
+template <int CW, bool BIG>
 struct UnitChannels {
-    static constexpr int value = CW == 8 ? 2 : (CW == 4 ? 4 : 8);
+    static constexpr int value = CW == 8 ? (BIG ? 4 : 2) : (CW == 4 ? (BIG ? 8 : 4) : 8);
 };
 
 // Work items handed to waves are runs of S units so that a wave's share of a
@@ -62,9 +67,10 @@ constexpr int kModeCounts = 0, kModeAffineAdd = 1, kModeAffineAddSign = 2;
 // write traffic) and wave priorities.  Measured: faster when a wave gets enough units (64 channels, 6 per wave:
 // 17.2 against 18.4 us; 128 channels, 12 per wave: 51 against 55 us), slower when it gets few (64 channels, 3 per
 // wave: 11.2 against 10.2 us; 128 channels, 3 per wave: 17.3 against 16.1 us).
+// For 256 and 512 input channels the flag selects the large-unit build instead (same residency).
 template <int CW, bool NARROW>
 struct Residency {
-    static constexpr int waves_per_simd = NARROW ? 4 : (CW == 1 ? 8 : CW == 2 ? 6 : CW == 4 ? 4 : 3);
+    static constexpr int waves_per_simd = CW == 8 ? 3 : CW == 4 ? 4 : NARROW ? 4 : (CW == 1 ? 8 : 6);
     static constexpr int window = (CW <= 2 && !NARROW) ? 16 : 32;
     static constexpr bool priorities = waves_per_simd <= 4;
 };
@@ -72,7 +78,7 @@ struct Residency {
 template <int CW, int MODE, bool NARROW>
 __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_per_simd)) void bconv3x3_kernel(const BconvArgs p) {
     constexpr int K32 = 18 * CW;
-    constexpr int Q = UnitChannels<CW>::value;
+    constexpr int Q = UnitChannels<CW, NARROW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     constexpr int WCH = Residency<CW, NARROW>::window;
     constexpr int WU = WCH / Q;  // units per staging window
@@ -361,7 +367,7 @@ static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 template <int CW, int MODE, bool NARROW>
 static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
-    constexpr int Q = UnitChannels<CW>::value;
+    constexpr int Q = UnitChannels<CW, NARROW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
@@ -377,7 +383,8 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
 }
 
 // Which kernel runs a problem of `tiles` 64-pixel tiles: 0 = the small-problem kernel (blocks split the depth),
-// 1 = the unit kernel at its wide residency, 2 = its NARROW build (64 and 128 input channels only).
+// 1 = the unit kernel at its wide residency, 2 = its second build: four waves per SIMD and whole-line stores for 64
+// and 128 input channels, units of twice the channels for 256 and 512.
 constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2;
 static int pick_build(long long tiles, int cin, int cout) {
     if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
@@ -385,6 +392,10 @@ static int pick_build(long long tiles, int cin, int cout) {
         // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (cout / 8);
         if (units >= (cin == 64 ? 4ll : 8ll) * simd_count() * 4) return kBuildNarrow;
+    } else {
+        // six large units or more per wave
+        const long long big_units = tiles * (cout / (cin == 256 ? 8 : 4));
+        if (cout % 8 == 0 && big_units >= 6ll * simd_count() * (cin == 256 ? 4 : 3)) return kBuildNarrow;
     }
     return kBuildWide;
 }
@@ -393,9 +404,7 @@ template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     const int build = pick_build(tiles, CW * 64, a.cout);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
-    if constexpr (CW <= 2) {
-        if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
-    }
+    if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
     return launch_variant<CW, MODE, false>(a, tiles, stream);
 }
 

@@ -162,8 +162,9 @@ DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
 /*
  * No counterpart in the reference: which of the three builds of the direct kernel dab_bconv3x3* runs for a problem of
  * n_out_pixels = N*OH*OW on the current device: 0 = the small-problem kernel (a block splits the depth over its
- * waves), 1 = the unit kernel at its wide residency, 2 = its four-waves-per-SIMD build (64 and 128 input channels,
- * many units per wave); -1 for shapes the direct kernel does not take.  For tests and tuning: a parity test names the
+ * waves), 1 = the unit kernel's build for mid-sized problems, 2 = its build for large ones (four waves per SIMD and
+ * whole-line stores for 64 and 128 input channels, units of twice the channels for 256 and 512; taken when a wave
+ * gets many units); -1 for shapes the direct kernel does not take.  For tests and tuning: a parity test names the
  * build it means to cover.
  */
 DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);

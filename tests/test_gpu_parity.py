@@ -282,6 +282,8 @@ def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, str
     (170, 28, 28, 128, 128, 1, 2), (44, 56, 56, 64, 64, 1, 2),
     # just below the switch: the wide build on nearly the same problem
     (160, 28, 28, 128, 128, 1, 1),
+    # 256 and 512 input channels: the builds with units of twice the channels, taken from six such units per wave on
+    (256, 14, 14, 256, 256, 1, 2), (200, 7, 7, 512, 512, 1, 2), (190, 14, 14, 256, 512, 2, 1),
 ])
 def test_fused_epilogues_of_the_named_build(dab, n, h, w, cin, cout, stride, build):
     """BinConv + Affine + Add (+ sign) through the build the test names (asked from the library, so the case cannot

@@ -270,7 +270,9 @@ def test_bireal18_batch256_matches_cpu(mods, stem):
     # the builds this configuration is there to cover
     assert capi.lib.dab_bconv3x3_build(batch * 56 * 56, 64, 64) == 2
     assert capi.lib.dab_bconv3x3_build(batch * 28 * 28, 128, 128) == 2
-    assert capi.lib.dab_bconv3x3_build(batch * 14 * 14, 256, 256) == 1
+    assert capi.lib.dab_bconv3x3_build(batch * 14 * 14, 256, 256) == 2
+    assert capi.lib.dab_bconv3x3_build(batch * 7 * 7, 512, 512) == 2
+    assert capi.lib.dab_bconv3x3_build(batch * 7 * 7, 256, 512) == 1
     gone = blobs_not_produced(n, layers)
     gen = torch.Generator().manual_seed(21)
     x = torch.randn((batch, 224, 224, 3), generator=gen).cuda()
