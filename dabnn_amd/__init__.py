@@ -17,6 +17,7 @@ from .ops import (  # noqa: F401
     bconv_3x3_affine_add,
     bconv_3x3_affine_add_sign,
     bgemm,
+    bgemm_overwrite,
     bitpack_nchw,
     col_row_words,
     concat,

@@ -51,6 +51,7 @@ SIGNATURES = {
     "dab_fused_binarize_im2col": (_i, [_vp] + [_i] * 12 + [_vp, _vp]),
     "dab_col_row_words": (_i, [_i, _i, _i]),
     "dab_bgemm": (_i, [_i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp]),
+    "dab_bgemm_overwrite": (_i, [_i, _i, _i, _vp, _i, _vp, _i, _vp, _i, _vp]),
     "dab_weight_transpose": (_i, [_vp, _i, _i, _vp, _vp]),
     "dab_bconv3x3": (_i, [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp]),
     "dab_bconv3x3_affine_add": (_i, [_vp, _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

@@ -33,6 +33,7 @@ struct BgemmArgs {
     int n_runs;  // ceil(n / Q) column runs per row tile
     int items_per_wave, items_extra;
     FastDiv div_runs;
+    int overwrite;  // C = counts instead of C += counts: what the reference's fill(0) + bgemm pair leaves in C
 };
 
 constexpr int kGemmWavesPerBlock = 4;
@@ -42,13 +43,14 @@ constexpr int kChunk = 8;  // K words per chunk of the generic variant
 // (shifted) run and are skipped; the test is wave-uniform.
 template <int Q>
 __device__ __forceinline__ void add_to_c(float *__restrict__ c, int ldc, int row, bool row_ok, int j0, int j_first,
-                                         const uint32_t (&acc)[Q]) {
+                                         const uint32_t (&acc)[Q], bool overwrite) {
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const int j = j0 + q;
         if (j >= j_first && row_ok) {
             float *d = c + (size_t)j * ldc + row;
-            *d += __uint_as_float(acc[q]) - kAccBias;
+            const float cnt = __uint_as_float(acc[q]) - kAccBias;
+            *d = overwrite ? cnt : *d + cnt;  // 0.f + cnt == cnt: the store alone is the fill + accumulate pair
         }
     }
 }
@@ -97,8 +99,8 @@ __global__ __launch_bounds__(64 * kGemmWavesPerBlock, K64R >= 72 ? 3 : (K64R >= 
         const int j_first = run * Q;
         const int j0 = j_first + Q <= p.n ? j_first : p.n - Q;
         uint32_t acc[Q];
-        unit_rowmajor<K32, Q, 2>(p.b + (size_t)j0 * K64R, w, acc);  // B streams through the scalar cache: two vectors per wait
-        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
+        unit_rowmajor<K32, Q, 2, (K64R >= 72)>(p.b + (size_t)j0 * K64R, w, acc);  // B streams through the scalar cache: two vectors per wait
+        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc, p.overwrite != 0);
         if (++run == p.n_runs) {
             run = 0;
             ++mt;
@@ -174,7 +176,7 @@ __global__ __launch_bounds__(64 * kGemmWavesPerBlock) void bgemm_chunked_kernel(
                 acc[q] += __builtin_popcount(wlo ^ (uint32_t)bw) + __builtin_popcount(whi ^ (uint32_t)(bw >> 32));
             }
         }
-        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc);
+        add_to_c<Q>(p.c, p.ldc, row, row_ok, j0, j_first, acc, p.overwrite != 0);
         if (++run == p.n_runs) {
             run = 0;
             ++mt;
@@ -190,7 +192,8 @@ __global__ void bgemm_small_n_kernel(const BgemmArgs p) {
     const long long j = idx / p.m;
     uint32_t cnt = 0;
     for (int h = 0; h < p.k; ++h) cnt += __popcll(p.a[(size_t)h * p.lda + i] ^ p.b[(size_t)j * p.ldb + h]);
-    p.c[(size_t)j * p.ldc + i] += (float)cnt;
+    float *d = p.c + (size_t)j * p.ldc + i;
+    *d = p.overwrite ? (float)cnt : *d + (float)cnt;
 }
 
 template <int Q, class Kernel>
@@ -218,8 +221,8 @@ static int launch_resident(BgemmArgs &g, hipStream_t stream) {
 
 }  // namespace dab
 
-extern "C" int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c, int ldc,
-                         dab_stream_t stream) {
+static int bgemm_impl(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c, int ldc,
+                      bool overwrite, dab_stream_t stream) {
     using namespace dab;
     DAB_REQUIRE(a && b && c, "dab_bgemm: null pointer");
     DAB_REQUIRE(m > 0 && n > 0 && k > 0, "dab_bgemm: m %d n %d k %d", m, n, k);
@@ -235,6 +238,7 @@ extern "C" int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const 
     g.a = a, g.b = b, g.c = c;
     g.m = m, g.n = n, g.k = k;
     g.lda = lda, g.ldb = ldb, g.ldc = ldc;
+    g.overwrite = overwrite ? 1 : 0;
     hipStream_t s = as_stream(stream);
     if (n < 8) {
         const long long total = (long long)m * n;
@@ -255,4 +259,14 @@ extern "C" int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const 
     hipLaunchKernelGGL(bgemm_chunked_kernel, dim3(n_waves / kGemmWavesPerBlock), dim3(64 * kGemmWavesPerBlock), 0, s, g);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
+}
+
+extern "C" int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c, int ldc,
+                         dab_stream_t stream) {
+    return bgemm_impl(m, n, k, a, lda, b, ldb, c, ldc, false, stream);
+}
+
+extern "C" int dab_bgemm_overwrite(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c,
+                                   int ldc, dab_stream_t stream) {
+    return bgemm_impl(m, n, k, a, lda, b, ldb, c, ldc, true, stream);
 }

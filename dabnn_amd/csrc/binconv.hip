@@ -33,7 +33,6 @@ static int static_scratch(void **out) {
     return DAB_OK;
 }
 
-int fill_f32(float *x, long long total, float v, hipStream_t s);
 
 static bool direct_ok(int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int cout) {
     // dabnn/layers/BinConv.cpp:100-126: 3x3, equal strides, 64/128/256/512 input channels
@@ -84,11 +83,10 @@ extern "C" int dab_binconv_forward(const float *x, int n, int h, int w, int c, c
     uint64_t *col = static_cast<uint64_t *>(workspace);
     const long long npix = (long long)n * oh * ow;
     if (npix >= (1ll << 31)) return fail(DAB_EUNSUPPORTED, "dab_binconv_forward: too many output pixels");
-    int rc = fill_f32(out, npix * cout, 0.f, as_stream(stream));  // output_mat->fill<float>(0.f), BinConv.cpp:153
+    // output_mat->fill<float>(0.f) and the accumulation into it (BinConv.cpp:153-165) are one store: 0.f + count == count
+    int rc = dab_fused_binarize_im2col(x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, 1, 1, col, stream);
     if (rc != DAB_OK) return rc;
-    rc = dab_fused_binarize_im2col(x, n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, 1, 1, col, stream);
-    if (rc != DAB_OK) return rc;
-    rc = dab_bgemm(cout, (int)npix, hwc_words, wgt_t, cout, col, row_words, out, cout, stream);
+    rc = dab_bgemm_overwrite(cout, (int)npix, hwc_words, wgt_t, cout, col, row_words, out, cout, stream);
     if (rc == DAB_OK && method_out) *method_out = 1;
     return rc;
 }

@@ -122,8 +122,8 @@ void BinConv::forward_impl() const {
             break;
         }
         case BGEMM: {
-            // fill + fused_binarize_im2col + bgemm, dabnn/layers/BinConv.cpp:152-165
-            dab_check(dab_fill_f32(out, (int64_t)output_mat->total(), 0.f, s));
+            // fill + fused_binarize_im2col + bgemm, dabnn/layers/BinConv.cpp:152-165; the fill and the accumulation
+            // into it are one store (0.f + count == count)
             auto *col = static_cast<uint64_t *>(col_mat->dev);
             dab_check(dab_fused_binarize_im2col(x, n, h, w, c, kernel_h(), kernel_w(), pad_h, pad_w, stride_h, stride_w, 1,
                                                 1, col, s));
@@ -131,8 +131,8 @@ void BinConv::forward_impl() const {
             const int cols = n * output_mat->h * output_mat->w;
             const int k = (int)(weight_mat->total() / m);
             const int ldb = dab_col_row_words(kernel_h(), kernel_w(), c);  // rows are padded to 128 bits
-            dab_check(dab_bgemm(m, cols, k, static_cast<const uint64_t *>(transposed_weight_mat->dev), m, col, ldb, out, m,
-                                s));
+            dab_check(dab_bgemm_overwrite(m, cols, k, static_cast<const uint64_t *>(transposed_weight_mat->dev), m, col, ldb,
+                                          out, m, s));
             break;
         }
     }

@@ -122,6 +122,17 @@ def bgemm(m, n, k, a, lda, b, ldb, c, ldc):
     return c
 
 
+def bgemm_overwrite(m, n, k, a, lda, b, ldb, c, ldc):
+    """fill(0) + bgemm (dabnn/layers/BinConv.cpp:153-165) as one launch: C = popcount(A ^ B), C is not read."""
+    _need(a, torch.int64, "a")
+    _need(b, torch.int64, "b")
+    _need(c, torch.float32, "c")
+    if a.numel() < (k - 1) * lda + m or b.numel() < (n - 1) * ldb + k or c.numel() < (n - 1) * ldc + m:
+        raise capi.DabError(capi.DAB_EINVAL, "bgemm: operand smaller than its m/n/k/ld description")
+    check(lib.dab_bgemm_overwrite(m, n, k, _ptr(a), lda, _ptr(b), ldb, _ptr(c), ldc, _stream()))
+    return c
+
+
 def bconv_3x3(x, weight, stride=1, pad=1):
     """pad + bconv_3x3 (dabnn/bconv.h:855-931): packed [N,H,W,CW], weight int64 [Cout, 9*CW] -> fp32 counts."""
     _need(x, torch.int64, "x")

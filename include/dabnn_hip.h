@@ -109,6 +109,14 @@ DAB_API int dab_bgemm(int m, int n, int k, const uint64_t *a, int lda, const uin
               dab_stream_t stream);
 
 /*
+ * What the reference's pair output_mat->fill<float>(0.f) + bgemm leaves in C (dabnn/layers/BinConv.cpp:153-165,
+ * 168-189): C(i,j) = float(popcount(A(i,h) ^ B(h,j))) summed over h, written without reading C.  Bit for bit the
+ * result of dab_fill_f32(c, 0) followed by dab_bgemm (0.f + count == count), in one launch and without the read of C.
+ */
+DAB_API int dab_bgemm_overwrite(int m, int n, int k, const uint64_t *a, int lda, const uint64_t *b, int ldb, float *c,
+                                int ldc, dab_stream_t stream);
+
+/*
  * Weight transpose done by the BinConv constructor for its bgemm method
  * (dabnn/layers/BinConv.cpp:59-76): wt[i*m + j] = w[j*k + i].
  */

@@ -156,6 +156,23 @@ def test_bgemm_leading_dimensions(dab, m, n, k, lda, ldb, ldc):
     np.testing.assert_array_equal(c.cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("m,n,k,lda,ldb,ldc", [(512, 49, 72, 512, 72, 512), (128, 784, 18, 128, 18, 128), (24, 70, 5, 31, 9, 28),
+                                               (72, 65, 25, 72, 25, 72), (16, 3, 9, 16, 9, 16), (40, 64, 36, 48, 36, 40)])
+def test_bgemm_overwrite_is_fill_then_bgemm(dab, m, n, k, lda, ldb, ldc):
+    """The pair output_mat->fill(0) + bgemm of dabnn/layers/BinConv.cpp:153-165 as one store: whatever C held before
+    (NaN included) is gone, elements outside the m x n window (leading-dimension padding) are untouched."""
+    a = rng(13).integers(0, 2**64, size=(k, lda), dtype=np.uint64)
+    b = rng(14).integers(0, 2**64, size=(n, ldb), dtype=np.uint64)
+    c0 = rng(15).standard_normal((n, ldc)).astype(np.float32)
+    c0[::3, ::5] = np.nan
+    want = c0.copy()
+    want[:, :m] = 0.0
+    orc.bgemm_naive(m, n, k, a, lda, b, ldb, want, ldc)
+    c = dev_f(c0)
+    dab.bgemm_overwrite(m, n, k, dev_u(a), lda, dev_u(b), ldb, c, ldc)
+    np.testing.assert_array_equal(c.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
 def test_bgemm_rejects_bad_arguments(dab):
     a = torch.zeros(16, dtype=torch.int64, device="cuda")
     c = torch.zeros(16, dtype=torch.float32, device="cuda")
