@@ -91,7 +91,7 @@ struct BandOut {
 // A finished band (a wave's accumulators: 7 x 2 tiles of 16 pixels x 16 channels, wave (wm, wn) = pixels 112*wm ..,
 // channels 32*wn ..) goes through LDS to the pooled tensor, the carry and the sign bits.  All threads of the block
 // call it after a barrier that ended every other use of `stage`.
-template <bool SIGN, int SLOTS>
+template <bool SIGN, int SLOTS, int ROWS = 0>
 __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *stage, const f32x4v (&acc)[7][2], const BandOut o,
                                               int tid, int wm, int wn, int f_s, int f_i, float4 (&keep)[SLOTS],
                                               bool fold, bool write_carry) {
@@ -152,8 +152,11 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
         const float *col1 = &stage[(2 * px) * kStageStride + c4 * 4];
         const float4 lowest = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
         float4 prev = fold ? keep[slot] : lowest, even = lowest;
-        for (int r = 0; r < p.band_rows; ++r) {
-            const int ro = r * p.ow * kStageStride;
+        // ROWS: the band's rows when the kernel knows them (all loads of a column are then asked for at once)
+        const int rows = ROWS ? ROWS : p.band_rows, ow = ROWS ? kBandPixels / ROWS : p.ow;
+#pragma unroll
+        for (int r = 0; r < rows; ++r) {
+            const int ro = r * ow * kStageStride;
             const float4 h = max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
                                   *reinterpret_cast<const float4 *>(col1 + ro + kStageStride));
             if (r & 1) {
@@ -342,29 +345,46 @@ __global__ __launch_bounds__(kBandThreads) void fconv_maxpool_kernel(const Fconv
 }
 
 // The ImageNet stem itself -- 7x7, stride 2, pad 3 on three-channel images whose output is 112 pixels wide -- without
-// an im2col stage: a band's 13 input rows go to LDS as they are (229 pixels from x = -3, zeros outside the image), and
+// an im2col stage: a band's 13 input rows go to LDS as they are (230 pixels from x = -3, zeros outside the image), and
 // the matrix-core operands are read straight from them.  Wave (wm, wn) owns output row wm of the band and 32
-// channels; an output pixel's 21 values of one kernel row are contiguous (tile floats 6*ox + k', k' = 3*tx + ch),
-// so for every kernel row a lane's operand addresses are one base plus constants: depth slot s of the instruction
-// takes k' = 4s .. 4s+3 in four instructions, then k' = 16 + s in a fifth, and the seven k' = 20 of all kernel rows
-// fill two more (slot s = kernel row s, then 4 + s; the eighth slot's weight is zero).  148 depths for 147.  The
-// block's 64 filters sit in LDS in that order for all of its bands; the next band's rows are fetched into registers
-// while the current one is multiplied.
-constexpr int kTileStride = 688;                    // floats per tile row: 229 pixels x 3, rounded up to even
-constexpr int kTileRows = 13, kTilePixels = 229;
+// channels; an output pixel's 21 values of one kernel row are contiguous (tile elements 6*ox + k', k' = 3*tx + ch),
+// so a lane's operand addresses are a base plus constants.
+//
+// The products run on the bf16 matrix cores with fp32 accuracy (split operands, six v_mfma_f32_16x16x32_bf16 per 32
+// depths; common.h): the instruction takes 19 cycles where the eight fp32 ones for the same depth take 256.  The tile
+// is split once, on its way into LDS, into three planes of bf16 (hi, mid, lo); the filters stay fp32 in LDS and are
+// split when a wave reads them, once per band and depth group.  The cross terms need hi with non-finite values taken
+// out (common.h); a band with an infinity or a NaN in its rows -- a flag in LDS says so -- takes a second copy of the
+// loop that derives it from hi in registers, all other bands use hi as it is.  A depth group is
+// four slots of eight depths, slot g = lane / 16; the 147 depths make 19 slots: q = 0..13: kernel row q / 2, k' = 0..7
+// or 8..15; q = 14..17: k' = 16..19 of kernel rows (0, 1), (2, 3), (4, 5), (6, none); q = 18: k' = 20 of the seven
+// kernel rows, which a second small array per plane holds transposed (T20[ox][tile row]) so that they are contiguous
+// too; q = 19 is empty.  Empty halves read a zero area of the plane; the eighth element of slot 18 is masked (it is a
+// real tile value, and zero times an infinity would be a NaN).  160 depths for 147, five groups.
+// The block's 64 filters sit in LDS for all of its bands; the next band's rows are fetched into registers while the
+// current one is pooled.
+constexpr int kTileStride = 692;                    // elements per tile row: 115 pixel pairs x 6, + 2
+constexpr int kTileRows = 13, kTilePairs = 115;
+constexpr int kPlaneZero = 9000;                    // eight zeros behind the 13 x 692 tile elements
+constexpr int kPlaneT20 = kPlaneZero + 8;           // [112 output columns][16]: tile rows of element 6 * ox + 20
+constexpr int kPlane = kPlaneT20 + 112 * 16;        // bf16 elements per plane
 constexpr int kFilterStride = 148;                  // 7 x (16 + 4) + 7 + 1 floats per filter
 constexpr int kFilterFloats = kBandChannels * kFilterStride;
-constexpr int kStemLdsFloats = kFilterFloats + kBandPixels * kStageStride;  // the tile shares the staged band's space
-constexpr int kTileLoads = (kTileRows * kTilePixels + kBandThreads - 1) / kBandThreads;
+constexpr int kStemLdsFloats = kFilterFloats + kBandPixels * kStageStride;  // the planes share the staged band's space
+constexpr int kPairLoads = (kTileRows * kTilePairs + kBandThreads - 1) / kBandThreads;
 constexpr int kStemKeepSlots = 2;  // 56 pooled columns x 16 channel groups on 512 threads
 static_assert(56 * 16 <= kStemKeepSlots * kBandThreads, "pooled columns of the stem");
+static_assert(kTileStride * kTileRows <= kPlaneZero && (kPlaneT20 * 2) % 16 == 0 && (kPlane * 2) % 16 == 0, "plane layout");
+static_assert(3 * kPlane * 2 <= kBandPixels * kStageStride * 4, "the three planes fit the staged band's space");
 
 template <bool SIGN>
 __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const FconvPoolArgs p) {
     constexpr int BN = kBandChannels, TM = 7, TN = 2;
-    static_assert(kTileStride * kTileRows <= kBandPixels * kStageStride, "the tile fits the staged band's space");
+    typedef uint32_t u32x2a __attribute__((ext_vector_type(2), aligned(4)));
     __shared__ __attribute__((aligned(16))) float smem[kStemLdsFloats];
-    float *const wl = smem, *const tile = smem + kFilterFloats;
+    float *const wl = smem, *const stage = smem + kFilterFloats;
+    uint16_t *const planes = reinterpret_cast<uint16_t *>(stage);  // hi, mid, lo: kPlane elements each
+    __shared__ int special_flag;  // the band's rows hold an infinity or a NaN
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -378,19 +398,27 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
     for (int slot = 0; slot < kStemKeepSlots; ++slot) keep[slot] = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
     bool fold = false;
 
-    // the thread's pixels of a tile: byte offset from the tile's first row in the image, and place in LDS
-    uint32_t t_off[kTileLoads];
-    int t_lds[kTileLoads];
-#pragma unroll
-    for (int j = 0; j < kTileLoads; ++j) {
-        const int q = tid + kBandThreads * j;
-        const int ry = q / kTilePixels, cx = q - ry * kTilePixels, x = cx - 3;
-        const bool ok = q < kTileRows * kTilePixels && (unsigned)x < (unsigned)p.wd;
-        t_off[j] = ok ? (uint32_t)((ry * p.wd + x) * 12) : kPoolOob;
-        t_lds[j] = q < kTileRows * kTilePixels ? ry * kTileStride + cx * 3 : -1;
-    }
+    // the thread's pixel pairs of a tile (pair u = tid + 512 * j: tile row u / 115, pixels 2 * (u % 115) - 3 and the
+    // next): byte offsets from the tile's first row in the image and places in a plane, worked out again wherever
+    // they are needed rather than held in registers across the multiplication
+    struct PairPlace {
+        uint32_t off0, off1;
+        int lds, t20;
+    };
+    auto pair_place = [&](int j) {
+        int u = tid + kBandThreads * j;
+        asm volatile("" : "+v"(u));  // worked out here every time: hoisted out of the band loop these values are spilled
+        const int ry = u / kTilePairs, pr = u - ry * kTilePairs, x0 = 2 * pr - 3;
+        const bool in = u < kTileRows * kTilePairs;
+        PairPlace q;
+        q.off0 = in && (unsigned)x0 < (unsigned)p.wd ? (uint32_t)((ry * p.wd + x0) * 12) : kPoolOob;
+        q.off1 = in && (unsigned)(x0 + 1) < (unsigned)p.wd ? (uint32_t)((ry * p.wd + x0 + 1) * 12) : kPoolOob;
+        q.lds = in ? ry * kTileStride + 6 * pr : -1;
+        q.t20 = in && pr >= 3 ? kPlaneT20 + (pr - 3) * 16 + ry : -1;  // the pair's third element is tile element 6 * (pr - 3) + 20
+        return q;
+    };
     typedef float f32x3v __attribute__((ext_vector_type(3)));
-    f32x3v pf[kTileLoads];
+    f32x3v pf0[kPairLoads], pf1[kPairLoads];
     int img, band, row0, n0;
     auto enter = [&](int it) {
         const int bi = (int)p.div_ytiles.div((uint32_t)it);
@@ -406,20 +434,35 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         const auto x_rsrc = make_rsrc(p.x + (size_t)img * p.h * p.wd * 3, img_bytes);
         const uint32_t base = (uint32_t)((2 * row0 - 3) * p.wd * 12);
 #pragma unroll
-        for (int j = 0; j < kTileLoads; ++j)
-            pf[j] = __builtin_bit_cast(f32x3v, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, (int)(base + t_off[j]), 0, 0));
+        for (int j = 0; j < kPairLoads; ++j) {
+            const PairPlace q = pair_place(j);
+            pf0[j] = __builtin_bit_cast(f32x3v, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, (int)(base + q.off0), 0, 0));
+            pf1[j] = __builtin_bit_cast(f32x3v, __builtin_amdgcn_raw_buffer_load_b96(x_rsrc, (int)(base + q.off1), 0, 0));
+        }
     };
 
-    // lane constants of the operand reads (floats)
-    const int a_row = 2 * wm * kTileStride + 6 * f_i;
-    const float *pa = tile + a_row + 4 * f_s, *pa4 = tile + a_row + 16 + f_s;
-    const float *pa_l0 = tile + a_row + f_s * kTileStride + 20;
-    const float *pa_l1 = tile + a_row + (f_s < 3 ? 4 + f_s : 6) * kTileStride + 20;
-    const float *pb = wl + (wn * 32 + f_i) * kFilterStride + 4 * f_s, *pb4 = pb + 16 - 3 * f_s;
-    const float *pb_l = wl + (wn * 32 + f_i) * kFilterStride + 140 + f_s;
+    // lane constants of the operand reads: the plane elements of a slot's two halves of four (tile i of the wave's
+    // row: + 96 * i; slot 18: + 256 * i; the zero area: + 0) and the floats of the same depths in a filter.  Groups
+    // 0..2 and the first two slots of group 3 are eight consecutive k' of kernel row 2 * G + g / 2: group 0's
+    // offsets plus a constant.  The other slots of group 3 and group 4 have offsets of their own.
+    const int base_a = 2 * wm * kTileStride + 6 * f_i;
+    const int a_main = base_a + (f_s >> 1) * kTileStride + 8 * (f_s & 1), b_main = (f_s >> 1) * 20 + 8 * (f_s & 1);
+    // group 3: slots 12, 13 (kernel row 6), 14, 15 (k' = 16..19 of kernel rows (0, 1) and (2, 3))
+    const int a0_g3 = f_s < 2 ? a_main + 6 * kTileStride : base_a + 2 * (f_s - 2) * kTileStride + 16;
+    const int a1_g3 = a0_g3 + (f_s < 2 ? 4 : kTileStride);
+    const int b0_g3 = f_s < 2 ? b_main + 120 : 2 * (f_s - 2) * 20 + 16, b1_g3 = b0_g3 + (f_s < 2 ? 4 : 20);
+    // group 4: slots 16 (kernel rows 4, 5), 17 (row 6, nothing), 18 (k' = 20 of all rows), 19 (nothing)
+    const int a0_g4 = f_s < 2 ? base_a + (4 + 2 * f_s) * kTileStride + 16 : f_s == 2 ? kPlaneT20 + f_i * 16 + 2 * wm : kPlaneZero;
+    const int a1_g4 = f_s == 0 ? a0_g4 + kTileStride : f_s == 2 ? a0_g4 + 4 : kPlaneZero;
+    const int s0_g4 = f_s < 2 ? 96 : f_s == 2 ? 256 : 0, s1_g4 = f_s == 0 ? 96 : f_s == 2 ? 256 : 0;
+    const int b0_g4 = f_s < 2 ? (4 + 2 * f_s) * 20 + 16 : f_s == 2 ? 140 : 0, b1_g4 = f_s == 0 ? b0_g4 + 20 : f_s == 2 ? 144 : 0;
+    const bool b0_ok_g4 = f_s != 3, b1_ok_g4 = f_s == 0 || f_s == 2;
+    const uint32_t keep_g4 = f_s == 2 ? 0x0000ffffu : 0xffffffffu;  // slot 18: seven kernel rows, the eighth element out
 
     enter(item);
     fetch_tile();
+    if (tid == 0) special_flag = 0;
+    __syncthreads();
     int filters_of = -1;  // the channel tile whose filters are in LDS
     for (;;) {
         // here: the band's rows are in registers (or on their way), every thread is past its last read of the LDS
@@ -433,70 +476,101 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
                 wl[idx] = (co < rows_n && r < 147) ? p.w[(size_t)(n0 + co) * 147 + k] : 0.f;
             }
         }
+        if (tid < 12) reinterpret_cast<uint32_t *>(planes + (tid >> 2) * kPlane + kPlaneZero)[tid & 3] = 0u;
+        bool any_special = false;
 #pragma unroll
-        for (int j = 0; j < kTileLoads; ++j)
-            if (t_lds[j] >= 0) {
-                tile[t_lds[j]] = pf[j][0], tile[t_lds[j] + 1] = pf[j][1], tile[t_lds[j] + 2] = pf[j][2];
+        for (int j = 0; j < kPairLoads; ++j) {
+            const PairPlace q = pair_place(j);
+            if (q.lds >= 0) {
+                const SplitParts s[6] = {split_bf16x3(pf0[j][0]), split_bf16x3(pf0[j][1]), split_bf16x3(pf0[j][2]),
+                                         split_bf16x3(pf1[j][0]), split_bf16x3(pf1[j][1]), split_bf16x3(pf1[j][2])};
+                uint32_t *d = reinterpret_cast<uint32_t *>(planes + q.lds);
+#pragma unroll
+                for (int e = 0; e < 6; ++e) any_special |= s[e].hif != s[e].hi;
+#pragma unroll
+                for (int e = 0; e < 3; ++e) {
+                    d[e] = pack_upper_halves(s[2 * e].hi, s[2 * e + 1].hi);
+                    d[kPlane / 2 + e] = pack_upper_halves(s[2 * e].mid, s[2 * e + 1].mid);
+                    d[2 * (kPlane / 2) + e] = pack_upper_halves(s[2 * e].lo, s[2 * e + 1].lo);
+                }
+                if (q.t20 >= 0) {
+                    planes[q.t20] = (uint16_t)(s[2].hi >> 16);
+                    planes[kPlane + q.t20] = (uint16_t)(s[2].mid >> 16);
+                    planes[2 * kPlane + q.t20] = (uint16_t)(s[2].lo >> 16);
+                }
             }
+        }
+        if (any_special) special_flag = 1;
         __syncthreads();
 
         const BandOut o{img, band, row0, n0, n0 / BN};
         const int next = item + range.step;
         const bool has_next = next < range.end;
-        if (has_next) {
-            enter(next);
-            fetch_tile();
-        }
 
         f32x4v acc[TM][TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) acc[i][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+        // a slot's eight bf16 of every plane: two halves of four (each 4-byte aligned)
+        auto a_frag = [&](auto derive_finite, int e0, int e1, uint32_t keep_mask) {
+            SplitFrag8 f;
+            const u32x2a h0 = *reinterpret_cast<const u32x2a *>(planes + e0), h1 = *reinterpret_cast<const u32x2a *>(planes + e1);
+            const u32x2a m0 = *reinterpret_cast<const u32x2a *>(planes + kPlane + e0), m1 = *reinterpret_cast<const u32x2a *>(planes + kPlane + e1);
+            const u32x2a l0 = *reinterpret_cast<const u32x2a *>(planes + 2 * kPlane + e0), l1 = *reinterpret_cast<const u32x2a *>(planes + 2 * kPlane + e1);
+            f.hi = SplitFrag8::u4{h0.x, h0.y, h1.x, h1.y & keep_mask};
+            f.mid = SplitFrag8::u4{m0.x, m0.y, m1.x, m1.y & keep_mask};
+            f.lo = SplitFrag8::u4{l0.x, l0.y, l1.x, l1.y & keep_mask};
+            if constexpr (decltype(derive_finite)::value) {
 #pragma unroll
-        for (int ty = 0; ty < 7; ++ty) {
-            float2 alo[TM], ahi[TM];
-            float a4[TM];
-            float4 b[TN];
-            float b4[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                alo[i] = *reinterpret_cast<const float2 *>(pa + ty * kTileStride + 96 * i);
-                ahi[i] = *reinterpret_cast<const float2 *>(pa + ty * kTileStride + 96 * i + 2);
-                a4[i] = pa4[ty * kTileStride + 96 * i];
+                for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
+            } else {
+                f.hif = f.hi;
             }
+            return f;
+        };
+        auto b_frag = [&](int j, int e0, int e1, bool ok0, bool ok1) {
+            const float *row = wl + (wn * 32 + j * 16 + f_i) * kFilterStride;
+            const float4 v0 = *reinterpret_cast<const float4 *>(row + e0), v1 = *reinterpret_cast<const float4 *>(row + e1);
+            const float x[8] = {ok0 ? v0.x : 0.f, ok0 ? v0.y : 0.f, ok0 ? v0.z : 0.f, ok0 ? v0.w : 0.f,
+                                ok1 ? v1.x : 0.f, ok1 ? v1.y : 0.f, ok1 ? v1.z : 0.f, ok1 ? v1.w : 0.f};
+            SplitFrag8 f;
+            f.set(x);
+            return f;
+        };
+        auto multiply = [&](auto derive_finite) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) {
-                b[j] = *reinterpret_cast<const float4 *>(pb + ty * 20 + j * 16 * kFilterStride);
-                b4[j] = pb4[ty * 20 + j * 16 * kFilterStride];
+            for (int G = 0; G < 5; ++G) {
+                SplitFrag8 b[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    b[j] = G < 3    ? b_frag(j, b_main + 40 * G, b_main + 40 * G + 4, true, true)
+                           : G == 3 ? b_frag(j, b0_g3, b1_g3, true, true)
+                                    : b_frag(j, b0_g4, b1_g4, b0_ok_g4, b1_ok_g4);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const SplitFrag8 a =
+                        G < 3    ? a_frag(derive_finite, a_main + 2 * G * kTileStride + 96 * i, a_main + 2 * G * kTileStride + 96 * i + 4, 0xffffffffu)
+                        : G == 3 ? a_frag(derive_finite, a0_g3 + 96 * i, a1_g3 + 96 * i, 0xffffffffu)
+                                 : a_frag(derive_finite, a0_g4 + s0_g4 * i, a1_g4 + s1_g4 * i, keep_g4);
+                    mfma6_16x16x32(acc[i][0], acc[i][1], a, b[0], b[1]);
+                }
             }
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(alo[i].x, b[j].x, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(alo[i].y, b[j].y, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ahi[i].x, b[j].z, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(ahi[i].y, b[j].w, acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[i], b4[j], acc[i][j], 0, 0, 0);
-                }
+        };
+        if (__builtin_amdgcn_readfirstlane(special_flag) != 0)
+            multiply(std::true_type{});
+        else
+            multiply(std::false_type{});
+        int tid_band = tid;
+        asm volatile("" : "+v"(tid_band));  // the epilogue's addresses are worked out per band, not held (spilled) across the loop
+        // the next band's rows come while this band is pooled (their registers are free of the multiplication)
+        if (has_next) {
+            enter(next);
+            fetch_tile();
         }
-        {
-            float al0[TM], al1[TM], bl0[TN], bl1[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) al0[i] = pa_l0[96 * i], al1[i] = pa_l1[96 * i];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) bl0[j] = pb_l[j * 16 * kFilterStride], bl1[j] = pb_l[4 + j * 16 * kFilterStride];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(al0[i], bl0[j], acc[i][j], 0, 0, 0);
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(al1[i], bl1[j], acc[i][j], 0, 0, 0);
-                }
-        }
-        __syncthreads();  // the tile is dead: the staged band takes its place
-        band_epilogue<SIGN, kStemKeepSlots>(p, tile, acc, o, tid, wm, wn, f_s, f_i, keep, fold && o.band > 0, !p.chained || !has_next);
+        __syncthreads();  // the planes are dead: the staged band takes their place
+        if (tid == 0) special_flag = 0;  // the next band's rows set it again, after the barrier that ends this pass
+        band_epilogue<SIGN, kStemKeepSlots, 4>(p, stage, acc, o, tid_band, wm, wn, f_s, f_i, keep, fold && o.band > 0, !p.chained || !has_next);
         if (!has_next) break;
         fold = p.chained != 0;
         item = next;
