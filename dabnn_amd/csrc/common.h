@@ -35,6 +35,13 @@ inline hipStream_t as_stream(dab_stream_t s) { return reinterpret_cast<hipStream
 
 // Number of SIMDs on the current device (4 per CU); cached.
 int simd_count();
+// fconv_c32.hip: the 3x3, stride 1, 32-input-channel float convolution on the bf16 matrix cores; 1 = done, 0 = not its
+// shapes (the caller takes the general kernel), negative = error.
+bool fconv_c32_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
+                     int dil_w, int cout, int oh, int ow);
+int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias, const float *aff_a,
+                  const float *aff_b, int relu, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
+                  int dil_w, int cout, int oh, int ow, float *out, hipStream_t s);
 
 // Output extent of a convolution / pooling window (common/Shaper.cpp:34-54).
 inline int out_dim(int in, int pad, int k, int dil, int stride) { return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1; }
@@ -114,6 +121,37 @@ __device__ __forceinline__ SplitParts split_bf16x3(float x) {
 // the upper halves of two dwords as one: a in the lower 16 bits, b in the upper
 __device__ __forceinline__ uint32_t pack_upper_halves(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
+// The same split for a pair of finite values with the hardware's round-to-nearest conversions (v_cvt_pk_bf16_f32
+// packs two): hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid), both subtractions and the last conversion
+// exact.  5.5 vector instructions per value against about 10 for the truncating form with its tests.  An infinity or a
+// NaN would come out as NaN in mid and lo: callers check with bf16_pair_max / bf16_pairs_finite and take the
+// truncating form for the rare group that holds one.
+typedef __bf16 bf16x2v __attribute__((ext_vector_type(2)));
+typedef float f32x2v __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2v __attribute__((ext_vector_type(2)));
+struct SplitPair {
+    uint32_t hi, mid, lo;  // two bf16 each, the first value in the lower half
+};
+__device__ __forceinline__ SplitPair split_pair_finite(float x0, float x1) {
+    auto widen = [](uint32_t w) { return f32x2v{__builtin_bit_cast(float, w << 16), __builtin_bit_cast(float, w & 0xffff0000u)}; };
+    const f32x2v x = {x0, x1};
+    SplitPair s;
+    s.hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2v));
+    const f32x2v r = x - widen(s.hi);
+    s.mid = __builtin_bit_cast(uint32_t, __builtin_convertvector(r, bf16x2v));
+    const f32x2v r2 = r - widen(s.mid);
+    s.lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(r2, bf16x2v));
+    return s;
+}
+// Running maximum of the magnitudes of bf16 pairs (as 16-bit integers, half by half), and the test of the result.
+__device__ __forceinline__ uint32_t bf16_pair_max(uint32_t running, uint32_t pair) {
+    const u16x2v a = __builtin_bit_cast(u16x2v, running), b = __builtin_bit_cast(u16x2v, pair & 0x7fff7fffu);
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(a, b));
+}
+__device__ __forceinline__ bool bf16_pairs_finite(uint32_t running) {
+    return (running & 0xffffu) < 0x7f80u && (running >> 16) < 0x7f80u;
+}
+
 // Two bf16 in a dword, each replaced by zero when it is an infinity or a NaN.
 __device__ __forceinline__ uint32_t finite_bf16_pair(uint32_t w) {
     const uint32_t lo_ok = (w & 0x00007f80u) != 0x00007f80u ? 0x0000ffffu : 0u;
@@ -125,6 +163,17 @@ __device__ __forceinline__ uint32_t finite_bf16_pair(uint32_t w) {
 struct SplitFrag8 {
     typedef uint32_t u4 __attribute__((ext_vector_type(4)));
     u4 hi, hif, mid, lo;
+    // finite values only (see split_pair_finite); hif = hi; returns the running magnitude maximum with these values in
+    __device__ __forceinline__ uint32_t set_finite(const float (&x)[8], uint32_t running) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const SplitPair s = split_pair_finite(x[2 * i], x[2 * i + 1]);
+            hi[i] = s.hi, mid[i] = s.mid, lo[i] = s.lo;
+            running = bf16_pair_max(running, s.hi);
+        }
+        hif = hi;
+        return running;
+    }
     __device__ __forceinline__ void set(const float (&x)[8]) {
         SplitParts s[8];
 #pragma unroll

@@ -677,6 +677,9 @@ extern "C" int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw
     // kernel gains a few per cent over full rounds and loses as much as the last round is empty (32 -> 64 channels at
     // 112 x 112, one pass against two launches: 127 / 128 us at 672 bands, 166 / 143 at 784, 166 / 166 at 896,
     // 205 / 187 at 1036): it runs when the last round leaves less than an eighth of all slots idle.
+    // 3x3 convolutions over 32 channels that are large enough for the split-operand kernel: that kernel and a separate
+    // MaxPool beat the one pass over im2col slices (32 -> 64 at 112 x 112, batch 256: 0.76 + 0.21 against 1.35 ms)
+    if (dab::fconv_c32_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b.oh, b.ow)) return 0;
     const long long blocks = (long long)n * b.bands * ((cout + dab::kBandChannels - 1) / dab::kBandChannels);
     const long long cus = dab::simd_count() / 4;
     if (dab::takes_raw_tile(c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, b)) return 2 * blocks > cus ? 1 : 0;

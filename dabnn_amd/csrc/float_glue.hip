@@ -582,6 +582,11 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
     const long long span_imgs = 128 / ((long long)a.oh * a.ow) + 2;
     if (span_imgs * h * w * c * 4 >= (1ll << 30) || 128ll * a.K * 4 >= (1ll << 30) || 128ll * cout * 4 >= (1ll << 30))
         return fail(DAB_EUNSUPPORTED, "%s: image, filter or channel count too large for 32-bit tile offsets", fn);
+    {
+        const int rc = fconv_c32_try(x, n, h, w, c, wgt, bias, aff_a, aff_b, relu, kh, kw, pad_h, pad_w, stride_h, stride_w,
+                                     dil_h, dil_w, cout, a.oh, a.ow, out, s);
+        if (rc != 0) return rc < 0 ? rc : DAB_OK;
+    }
     // without padding every tap of every window is inside the image and the bounds test is dropped
     const bool padded = pad_h != 0 || pad_w != 0 || (a.oh - 1) * stride_h + (kh - 1) * dil_h >= h ||
                         (a.ow - 1) * stride_w + (kw - 1) * dil_w >= w;

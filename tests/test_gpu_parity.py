@@ -448,6 +448,80 @@ def test_fconv_affine_relu_equals_separate_layers(dab, affine, relu, bias):
     np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * np.abs(want).max())
 
 
+@pytest.mark.parametrize("n,h,w,pad,cout,bias,affine,relu", [
+    (24, 112, 112, 1, 32, False, True, True),   # the three-convolution stem's second convolution
+    (22, 112, 112, 1, 64, True, False, False),  # its third
+    (99, 59, 46, 2, 32, True, True, False),     # 16 929 tiles of 16 pixels: the last work item is one tile, pad 2
+    (25, 114, 114, 0, 64, False, False, True),  # no padding
+])
+def test_fconv_3x3_over_32_channels_on_split_operands(dab, n, h, w, pad, cout, bias, affine, relu):
+    """3x3, stride 1 convolutions over 32 channels that are large enough take the kernel that multiplies on the bf16
+    matrix cores with operands split in three (fp32 accuracy): within the float tolerance of the CPU layers on a sample
+    of images and of a float64 convolution on all of them, exact on small integers, and an infinity or a NaN in the
+    image comes out where IEEE arithmetic puts it (zero times infinity included: a zero weight)."""
+    # the size gate of the kernel, seen through the one entry point that reports it: these shapes no longer take the
+    # one-pass convolution + MaxPool
+    if cout == 64 and pad == 1:
+        assert not dab.fconv_maxpool_pays(n, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
+        assert dab.fconv_maxpool_pays(18, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
+    r = rng(61)
+    x = r.standard_normal((n, h, w, 32)).astype(np.float32)
+    wgt = (r.standard_normal((cout, 3, 3, 32)) / 17).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32) if bias else None
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+
+    def gpu(x, wgt):
+        return dab.fconv_affine_relu(dev_f(x), dev_f(wgt), dev_f(bv) if bias else None, dev_f(a) if affine else None,
+                                     dev_f(b) if affine else None, relu, 3, 3, pad, pad, 1, 1)
+
+    def cpu(img, wgt):
+        y = orc.fconv(img, wgt, bv, 3, 3, pad, pad, 1, 1)
+        if affine:
+            y = orc.affine_inplace(y.copy(), a, b)
+        return np.maximum(y, 0) if relu else y
+
+    def f64(x, wgt):
+        y = torch.nn.functional.conv2d(torch.from_numpy(x).cuda().double().permute(0, 3, 1, 2),
+                                       torch.from_numpy(wgt).cuda().double().permute(0, 3, 1, 2), padding=pad)
+        if bias:
+            y = y + torch.from_numpy(bv).cuda().double().view(1, -1, 1, 1)
+        if affine:
+            y = y * torch.from_numpy(a).cuda().double().view(1, -1, 1, 1) + torch.from_numpy(b).cuda().double().view(1, -1, 1, 1)
+        if relu:
+            y = torch.where(y < 0, torch.zeros_like(y), y)  # std::max(v, 0.f): a NaN stays
+        return y.permute(0, 2, 3, 1).cpu().numpy()
+
+    got = gpu(x, wgt).cpu().numpy()
+    want = f64(x, wgt)
+    assert got.shape == want.shape
+    scale = np.abs(want).max()
+    np.testing.assert_allclose(got, want, rtol=RTOL, atol=RTOL * scale)
+    # much closer than the tolerance asks: the split loses nothing an fp32 loop keeps
+    assert np.abs(got - want).max() <= 4e-6 * scale
+    for i in (0, n // 2, n - 1):
+        np.testing.assert_allclose(got[i], cpu(x[i], wgt), rtol=RTOL, atol=RTOL * scale)
+    # small integers: every product and partial sum is exact
+    xi = r.integers(-3, 4, x.shape).astype(np.float32)
+    wi = r.integers(-2, 3, wgt.shape).astype(np.float32)
+    if affine:
+        a, b = r.integers(-2, 3, cout).astype(np.float32), r.integers(-9, 10, cout).astype(np.float32)
+    if bias:
+        bv = r.integers(-5, 6, cout).astype(np.float32)
+    goti = gpu(xi, wi).cpu().numpy()
+    for i in (0, n - 1):
+        np.testing.assert_array_equal(goti[i], cpu(xi[i], wi))
+    # a NaN pixel, an infinity in one channel, an infinity in a weight (its products with the image's zeros are NaN)
+    xi[0, h // 2, w // 3, :] = np.nan
+    xi[-1, h // 3, w // 2, 5] = np.inf
+    xi[1, 0, 0, 7] = -np.inf
+    wi[3, 1, 1, 9] = np.inf
+    with np.errstate(invalid="ignore"):
+        want = f64(xi, wi)
+    goti = gpu(xi, wi).cpu().numpy()
+    np.testing.assert_array_equal(np.isnan(goti), np.isnan(want))
+    np.testing.assert_array_equal(goti[~np.isnan(want)], want[~np.isnan(want)].astype(np.float32))
+
+
 def test_fconv_ramp_cases_of_reference_tests(dab):
     """tests/fconv_test.cpp:14-41 and :43-70: ramp image and ramp weights, exact in fp32."""
     for (h, k, pad, stride) in [(4, 3, 1, 1), (8, 5, 2, 2)]:
