@@ -27,7 +27,6 @@ struct FconvC32Args {
     uint32_t x_bytes;
     int tiles;          // 16-pixel tiles of the output: n * oh * ow / 16
     int items;          // groups of four tiles
-    int waves;          // persistent waves of the launch
     FastDiv div_tiles_per_row, div_oh;
     int tiles_per_row;
 };
@@ -68,9 +67,13 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
 
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, p.x_bytes);
     typedef float f32x4r __attribute__((ext_vector_type(4)));
-    const int wv = blockIdx.x * (kC32Threads / 64) + wave;
+    // A block works through a contiguous range of items, its waves side by side: the image rows above and below the
+    // ones it is on were fetched by the block itself a moment ago and are still in its L2 (with the items dealt to all
+    // waves in turn every row was fetched from memory twice, by blocks on different XCDs).
+    const int per = p.items / (int)gridDim.x, extra = p.items - per * (int)gridDim.x, b = (int)blockIdx.x;
+    const int first = b * per + (b < extra ? b : extra), last = first + per + (b < extra ? 1 : 0);
 
-    for (int item = wv; item < p.items; item += p.waves) {
+    for (int item = first + wave; item < last; item += kC32Threads / 64) {
         // the lane's pixel of each tile: byte offset of its window's first tap (may lie outside the image: then the
         // row or column test below sends the load out of range), and its coordinates for those tests
         int off0[PT], iy0[PT], ix0[PT];
@@ -97,14 +100,14 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
             }
         };
         // a filter fragment: output channels 16 * nt + f_i, depths 8 * g .. + 7 of the tap
-        auto filter_frag = [&](int nt, int tap) {
+        auto filter_frag = [&](auto filters_special, int nt, int tap) {
             const uint16_t *src = planes + (nt * 16 + f_i) * ROW + tap * 32 + 8 * g;
             SplitFrag8 f;
             f.hi = *reinterpret_cast<const SplitFrag8::u4 *>(src);
             f.mid = *reinterpret_cast<const SplitFrag8::u4 *>(src + PLANE);
             f.lo = *reinterpret_cast<const SplitFrag8::u4 *>(src + 2 * PLANE);
             f.hif = f.hi;
-            if (w_special) {
+            if constexpr (decltype(filters_special)::value) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
             }
@@ -119,6 +122,7 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
 
         f32x4r raw_lo[PT], raw_hi[PT];
         fetch(0, raw_lo, raw_hi);
+        auto all_taps = [&](auto filters_special) {
         // the taps one after the other (not unrolled: the compiler would otherwise start all nine taps' loads at once
         // and spill); the next tap's pixels are on their way while this tap is multiplied
 #pragma unroll 1
@@ -144,40 +148,54 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
             // rows of the product = output channels (the filter fragment), columns = pixels
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const SplitFrag8 f = filter_frag(nt, tap);
+                const SplitFrag8 f = filter_frag(filters_special, nt, tap);
                 mfma6_16x16x32(acc[0][nt], acc[1][nt], f, px[0], px[1]);
                 mfma6_16x16x32(acc[2][nt], acc[3][nt], f, px[2], px[3]);
             }
         }
+        };
+        if (w_special)
+            all_taps(std::true_type{});
+        else
+            all_taps(std::false_type{});
 
         // accumulator element e of lane l: output channel 16 * nt + 4 * (l / 16) + e of pixel l % 16
         auto store_all = [&]() {
 #pragma clang fp contract(off)
+            float bs[NT][4], as[NT][4], bb[NT][4];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            const int co = nt * 16 + 4 * g;
-            const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float bs[4] = {bias.x, bias.y, bias.z, bias.w}, as[4] = {fa.x, fa.y, fa.z, fa.w}, bb[4] = {fb.x, fb.y, fb.z, fb.w};
+            for (int nt = 0; nt < NT; ++nt) {
+                const int co = nt * 16 + 4 * g;
+                const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                bs[nt][0] = bias.x, bs[nt][1] = bias.y, bs[nt][2] = bias.z, bs[nt][3] = bias.w;
+                as[nt][0] = fa.x, as[nt][1] = fa.y, as[nt][2] = fa.z, as[nt][3] = fa.w;
+                bb[nt][0] = fb.x, bb[nt][1] = fb.y, bb[nt][2] = fb.z, bb[nt][3] = fb.w;
+            }
+            // a pixel's channel tiles one after the other: its 64-byte pieces complete 128-byte lines while they are
+            // still in the write path
 #pragma unroll
             for (int t = 0; t < PT; ++t) {
                 const int T = item * PT + t;
                 if (T >= p.tiles) continue;
-                float v[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    v[e] = acc[t][nt][e];
-                    if (p.bias) v[e] = v[e] + bs[e];
-                    if (p.aff_a) {
-                        const float prod = as[e] * v[e];
-                        v[e] = prod + bb[e];
+                for (int nt = 0; nt < NT; ++nt) {
+                    float v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = acc[t][nt][e];
+                        if (p.bias) v[e] = v[e] + bs[nt][e];
+                        if (p.aff_a) {
+                            const float prod = as[nt][e] * v[e];
+                            v[e] = prod + bb[nt][e];
+                        }
+                        if (p.relu) v[e] = v[e] < 0.f ? 0.f : v[e];  // std::max(v, 0.f): a NaN stays
                     }
-                    if (p.relu) v[e] = v[e] < 0.f ? 0.f : v[e];  // std::max(v, 0.f): a NaN stays
+                    *reinterpret_cast<float4 *>(p.out + ((size_t)T * 16 + f_i) * COUT + nt * 16 + 4 * g) =
+                        make_float4(v[0], v[1], v[2], v[3]);
                 }
-                *reinterpret_cast<float4 *>(p.out + ((size_t)T * 16 + f_i) * COUT + co) = make_float4(v[0], v[1], v[2], v[3]);
             }
-        }
         };
         store_all();
     }
@@ -212,7 +230,7 @@ int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, 
     a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.out = out, a.relu = relu;
     a.h = h, a.wd = w, a.oh = oh, a.ow = ow, a.cout = cout, a.pad_h = pad_h, a.pad_w = pad_w;
     a.x_bytes = (uint32_t)((long long)n * h * w * 128);
-    a.tiles = (int)tiles, a.items = (int)((tiles + kC32PixelTiles - 1) / kC32PixelTiles), a.waves = blocks * (kC32Threads / 64);
+    a.tiles = (int)tiles, a.items = (int)((tiles + kC32PixelTiles - 1) / kC32PixelTiles);
     a.tiles_per_row = ow / 16;
     a.div_tiles_per_row = FastDiv((uint32_t)a.tiles_per_row), a.div_oh = FastDiv((uint32_t)oh);
     if (cout == 32)
