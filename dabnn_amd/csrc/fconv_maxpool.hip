@@ -154,7 +154,8 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
         float4 prev = fold ? keep[slot] : lowest, even = lowest;
         // ROWS: the band's rows when the kernel knows them (all loads of a column are then asked for at once)
         const int rows = ROWS ? ROWS : p.band_rows, ow = ROWS ? kBandPixels / ROWS : p.ow;
-#pragma unroll
+        constexpr int kUnrollRows = ROWS > 0 ? ROWS : 1;
+#pragma unroll kUnrollRows
         for (int r = 0; r < rows; ++r) {
             const int ro = r * ow * kStageStride;
             const float4 h = max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
