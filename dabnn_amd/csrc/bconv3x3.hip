@@ -27,6 +27,7 @@ struct BconvArgs {
     int n_groups;  // cout / Q channel groups per tile
     int items_per_wave, items_extra;  // split of the work items over the waves
     uint32_t x_bytes;
+    int half;      // HALF kernels: which 512 of the 1024 input channels (0 or 1)
     FastDiv div_ow, div_oh, div_groups;
     // fused epilogue (MODE >= 1 kernels only): out = a*cnt + b (+ shortcut); MODE 2 also writes sign bits of out
     const float *epi_a;
@@ -59,6 +60,8 @@ struct ItemUnits {
 
 // MODE 0: raw counts.  1: + Affine (+ Add).  2: the same and a sign-packed copy of the result.
 constexpr int kModeCounts = 0, kModeAffineAdd = 1, kModeAffineAddSign = 2;
+// 3: out += counts, the second pass over a depth that is counted in two halves (1024 input channels)
+constexpr int kModeAccumulate = 3;
 
 // Resident waves per SIMD the kernel is built for, and the staging window that lets them fit the CU's LDS:
 // the activations take 18*CW VGPRs, so 64 and 128 channels leave room for 8 and 6 waves (with the 16-channel
@@ -75,9 +78,15 @@ struct Residency {
     static constexpr bool priorities = waves_per_simd <= 4;
 };
 
-template <int CW, int MODE, bool NARROW>
+// HALF: the tensors have 1024 channels (16 words per pixel and per filter tap) and the kernel counts one half of them,
+// words 8 * p.half .. + 7: the reference lists 1024 input channels as direct-convolution compatible
+// (dabnn/layers/BinConv.cpp:118); two passes of the 512-channel kernel, the second adding to the first's result.
+template <int CW, int MODE, bool NARROW, bool HALF = false>
 __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_per_simd)) void bconv3x3_kernel(const BconvArgs p) {
+    static_assert(!HALF || CW == 8, "halves of 1024 channels only");
     constexpr int K32 = 18 * CW;
+    constexpr int kPixelBytes = HALF ? 128 : CW * 8;       // one pixel's words
+    constexpr int kFilterWords = HALF ? 9 * 16 : 9 * CW;   // one output channel's words
     constexpr int Q = UnitChannels<CW, NARROW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     constexpr int WCH = Residency<CW, NARROW>::window;
@@ -104,11 +113,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
         // straight into the first 256 bytes of its own staging buffer, with no register and no wait involved; the
         // wave waits for it before it stages its first results there (by then the loads are long done: they were
         // issued before the activations the first unit has just used).
-        const uint32_t n_lines = ((uint32_t)(p.cout * 9 * CW * 8) + 127u) >> 7;
+        const uint32_t n_lines = ((uint32_t)(p.cout * kFilterWords * 8) + 127u) >> 7;
         const uint32_t first = (uint32_t)((blockIdx.x >> 3) * kWavesPerBlock + wib) * 64u;
         if (first < n_lines) {
             const uint32_t line = first + lane < n_lines ? first + lane : n_lines - 1;
-            const uint32_t last_byte = (uint32_t)(p.cout * 9 * CW * 8) - 4u;
+            const uint32_t last_byte = (uint32_t)(p.cout * kFilterWords * 8) - 4u;
             const uint32_t byte = line * 128u < last_byte ? line * 128u : last_byte;
             __builtin_amdgcn_global_load_lds(
                 (const void __attribute__((address_space(1))) *)(reinterpret_cast<const unsigned char *>(p.w) + byte),
@@ -128,6 +137,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             EpiAffineAddSign epi;
             epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
             epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
+            stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
+                                (slot * Q + Q - 1) >> 2, epi);
+        } else if constexpr (MODE == kModeAccumulate) {
+            EpiAccumulate epi;
+            epi.shortcut = p.out;
             stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
                                 (slot * Q + Q - 1) >> 2, epi);
         } else if constexpr (MODE == kModeAffineAdd) {
@@ -151,7 +165,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             const uint32_t n = p.div_oh.div(t);
             const int oy = t - n * p.OH;
             const int y0 = oy * p.stride - p.pad, x0 = ox * p.stride - p.pad;
-            const int base = ((n * p.H + y0) * p.W + x0) * (CW * 8);  // byte offset of tap (0,0); may be negative
+            // byte offset of tap (0,0); may be negative
+            const int base = ((n * p.H + y0) * p.W + x0) * kPixelBytes + (HALF ? p.half * 64 : 0);
 #pragma unroll
             for (int kh = 0; kh < 3; ++kh) {
                 const bool row_ok = (unsigned)(y0 + kh) < (unsigned)p.H;
@@ -159,7 +174,7 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
                 for (int kw = 0; kw < 3; ++kw) {
                     const bool ok = row_ok && (unsigned)(x0 + kw) < (unsigned)p.W;
                     // an offset beyond the descriptor's range reads as zero
-                    const int off = ok ? base + (kh * p.W + kw) * (CW * 8) : (int)0x80000000;
+                    const int off = ok ? base + (kh * p.W + kw) * kPixelBytes : (int)0x80000000;
                     uint32_t *dst = a + (kh * 3 + kw) * CW * 2;
                     if constexpr (CW == 1) {
                         const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, 0);
@@ -195,7 +210,8 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
         // epilogue and 256 or 512 input channels the memory pipes are busy with the shortcut and the filters are
         // large: there two vectors per wait win at batch 256 (51 against 59 us, 54 against 55; 0.4-0.7 us lost at
         // batch 64).
-        unit_rowmajor<K32, Q, ((MODE != kModeCounts && CW >= 4) ? 2 : 1)>(p.w + (size_t)cg * Q * (9 * CW), a, acc);
+        unit_rowmajor<K32, Q, ((MODE != kModeCounts && CW >= 4) ? 2 : 1), false, (HALF ? 128 : 0)>(
+            p.w + (size_t)cg * Q * kFilterWords + (HALF ? p.half * 8 : 0), a, acc);
         const int slot = cg % WU;
         if constexpr (kPrefetchFilters) {
             if (u == u0) __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the filter prefetch wrote into the staging buffer
@@ -365,19 +381,19 @@ static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
-template <int CW, int MODE, bool NARROW>
+template <int CW, int MODE, bool NARROW, bool HALF = false>
 static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW, NARROW>::value;
     constexpr int S = ItemUnits<Q, MODE == kModeAffineAddSign>::value;
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW>, 64 * kWavesPerBlock);
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW, HALF>, 64 * kWavesPerBlock);
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
     a.div_groups = FastDiv((uint32_t)a.n_groups);
-    hipLaunchKernelGGL((bconv3x3_kernel<CW, MODE, NARROW>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
+    hipLaunchKernelGGL((bconv3x3_kernel<CW, MODE, NARROW, HALF>), dim3(n_waves / kWavesPerBlock), dim3(64 * kWavesPerBlock), 0, stream, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }
@@ -419,7 +435,8 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     DAB_REQUIRE(stride > 0 && pad >= 0, "%s: stride %d pad %d", fn, stride, pad);
     DAB_REQUIRE(cin % 64 == 0, "%s: cin %d is not a multiple of 64", fn, cin);
     DAB_REQUIRE(h + 2 * pad >= 3 && w + 2 * pad >= 3, "%s: input smaller than the kernel", fn);
-    if (!(cin == 64 || cin == 128 || cin == 256 || cin == 512) || cout % 8 != 0)
+    const bool two_halves = cin == 1024 && mode == kModeCounts;  // no fused epilogue for 1024 input channels
+    if (!(cin == 64 || cin == 128 || cin == 256 || cin == 512 || two_halves) || cout % 8 != 0)
         return fail(DAB_EUNSUPPORTED, "%s: cin %d / cout %d not covered by the direct kernel", fn, cin, cout);
     DAB_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(wgt) & 7) == 0 &&
                     (reinterpret_cast<uintptr_t>(out) & 15) == 0,
@@ -453,6 +470,17 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     a.div_ow = FastDiv((uint32_t)a.OW), a.div_oh = FastDiv((uint32_t)a.OH);
     const long long tiles = (total + 63) / 64;
     hipStream_t s = as_stream(stream);
+    a.half = 0;
+    if (two_halves) {
+        // the 512-channel unit kernel on words 0..7 of every pixel and tap, then on words 8..15 adding to the result
+        // (the builds as for 512 channels; small problems take the unit kernel too)
+        const bool big = pick_build(tiles, 512, cout) == kBuildNarrow;
+        int rc = big ? launch_variant<8, kModeCounts, true, true>(a, tiles, s) : launch_variant<8, kModeCounts, false, true>(a, tiles, s);
+        if (rc != DAB_OK) return rc;
+        a.half = 1;
+        return big ? launch_variant<8, kModeAccumulate, true, true>(a, tiles, s)
+                   : launch_variant<8, kModeAccumulate, false, true>(a, tiles, s);
+    }
     switch (mode * 16 + cin / 64) {
         case kModeCounts * 16 + 1: return launch_bconv3x3<1, kModeCounts>(a, tiles, s);
         case kModeCounts * 16 + 2: return launch_bconv3x3<2, kModeCounts>(a, tiles, s);

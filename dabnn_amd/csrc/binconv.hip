@@ -35,9 +35,9 @@ static int static_scratch(void **out) {
 
 
 static bool direct_ok(int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int cout) {
-    // dabnn/layers/BinConv.cpp:100-126: 3x3, equal strides, 64/128/256/512 input channels
-    return kh == 3 && kw == 3 && stride_h == stride_w && pad_h == pad_w && (c == 64 || c == 128 || c == 256 || c == 512) &&
-           cout % 8 == 0;
+    // dabnn/layers/BinConv.cpp:100-126: 3x3, equal strides, 64/128/256/512/1024 input channels
+    return kh == 3 && kw == 3 && stride_h == stride_w && pad_h == pad_w &&
+           (c == 64 || c == 128 || c == 256 || c == 512 || c == 1024) && cout % 8 == 0;
 }
 }  // namespace dab
 

@@ -124,22 +124,25 @@ constexpr int kMaxCount = (1 << 23) - 1;
 // that no unit starts with a wait.  7.07 -> 6.88 cycles per pair for the bare unit body at four waves per SIMD, but
 // in the kernel the 16-32 SGPRs that then live across the store pass cost more than the wait: 97.9 against 95.7 us
 // for the seven batch-64 shapes.)
-template <int K32, int Q, int BV_WANTED = 1, bool GROUPED = false>
+// VEC_BYTES: distance between consecutive vectors in memory when they are not contiguous (one half of a filter row
+// that is twice as deep: every other 64 bytes); 0 = contiguous.
+template <int K32, int Q, int BV_WANTED = 1, bool GROUPED = false, int VEC_BYTES = 0>
 __device__ __forceinline__ void unit_rowmajor(const void *wbase, const uint32_t (&a)[K32], uint32_t (&acc)[Q]) {
     constexpr int D = Q * K32;
     constexpr int VW = D % 16 == 0 ? 16 : 8;
+    constexpr int VB = VEC_BYTES ? VEC_BYTES : VW * 4;
     constexpr int NV = D / VW;
     constexpr int BV = (NV % BV_WANTED == 0) ? BV_WANTED : 1;
     constexpr int NB = NV / BV;
     static_assert(K32 % 2 == 0 && D % VW == 0, "a dword pair never straddles two channels");
     typename SVec<VW>::type buf[2][BV];
     const uint32_t acc_init = kAccInit;  // the accumulators are written, not updated, by each channel's first pair
-    static_for<BV>([&](auto b_) { sload<VW, b_ * VW * 4>(buf[0][b_], wbase); });
+    static_for<BV>([&](auto b_) { sload<VW, b_ * VB>(buf[0][b_], wbase); });
     static_for<BV>([&](auto b_) { swait(buf[0][b_]); });
     static_for<NB>([&](auto j_) {
         constexpr int j = j_;
         if constexpr (j + 1 < NB)
-            static_for<BV>([&](auto b_) { sload<VW, ((j + 1) * BV + b_) * VW * 4>(buf[(j + 1) & 1][b_], wbase); });
+            static_for<BV>([&](auto b_) { sload<VW, ((j + 1) * BV + b_) * VB>(buf[(j + 1) & 1][b_], wbase); });
         static_for<BV>([&](auto b_) {
             static_for<VW / 2>([&](auto e_) {
                 constexpr int d = (j * BV + b_) * VW + e_ * 2;  // dword index within the Q-channel block
@@ -254,6 +257,19 @@ struct EpiAffineAdd {
         r.x = r.x + bv.x, r.y = r.y + bv.y, r.z = r.z + bv.z, r.w = r.w + bv.w;
         if constexpr (SC) r.x = r.x + sc.x, r.y = r.y + sc.y, r.z = r.z + sc.z, r.w = r.w + sc.w;
         return r;
+    }
+};
+// out = cnt + what out holds: the second half of a convolution whose depth is counted in two passes (counts are
+// integers far below 2^24, their float sum is exact)
+struct EpiAccumulate {
+    static constexpr bool kEmit = false;
+    static constexpr bool kShortcut = true;
+    const float *shortcut;  // = out
+    __device__ __forceinline__ void prepare(int) {}
+    template <bool SC>
+    __device__ __forceinline__ float4 apply(float4 v, float4 sc) const {
+        if constexpr (SC) v.x = v.x + sc.x, v.y = v.y + sc.y, v.z = v.z + sc.z, v.w = v.w + sc.w;
+        return v;
     }
 };
 struct EpiAffineAddSign : EpiAffineAdd {

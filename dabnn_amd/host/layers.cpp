@@ -83,10 +83,10 @@ BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad
 }
 
 bool BinConv::direct_conv_compatible() const {
-    // dabnn/layers/BinConv.cpp:100-126 (1024 input channels stay with bgemm here)
+    // dabnn/layers/BinConv.cpp:100-126
     const int c = input_mat->elem_c;
     return kernel_h() == 3 && kernel_w() == 3 && stride_h == stride_w && pad_h == pad_w &&
-           (c == 64 || c == 128 || c == 256 || c == 512) && weight_mat->n % 8 == 0;
+           (c == 64 || c == 128 || c == 256 || c == 512 || c == 1024) && weight_mat->n % 8 == 0;
 }
 
 BinConv::Method BinConv::method() const {

@@ -308,7 +308,9 @@ void Net::fuse_binconv_epilogues() {
     for (size_t i = 0; i < layers.size(); ++i) {
         auto bc = std::dynamic_pointer_cast<BinConv>(layers[i]);
         auto af = i + 1 < layers.size() ? std::dynamic_pointer_cast<Affine>(layers[i + 1]) : nullptr;
-        if (bc && af && bc->method() == BinConv::DIRECT_CONV && af->data_mat == bc->output_mat && bc->output_mat->c % 4 == 0) {
+        // (1024 input channels: the direct kernel counts them in two passes and has no fused epilogue)
+        if (bc && af && bc->method() == BinConv::DIRECT_CONV && bc->input_mat->elem_c <= 512 && af->data_mat == bc->output_mat &&
+            bc->output_mat->c % 4 == 0) {
             bc->fused_a = af->a_mat;
             bc->fused_b = af->b_mat;
             size_t skip = 1;

@@ -129,8 +129,10 @@ DAB_API int dab_weight_transpose(const uint64_t *w, int m, int k, uint64_t *wt, 
  * activation [n][h][w][cin/64]; taps outside the image read a zero word.
  * wgt is [cout][9*cin/64] words.  out is fp32 [n][oh][ow][cout] holding the
  * mismatch counts, oh = (h + 2*pad - 3)/stride + 1.
- * Implemented for cin in {64, 128, 256, 512} and cout % 8 == 0; other shapes
- * return DAB_EUNSUPPORTED (use dab_fused_binarize_im2col + dab_bgemm, as the
+ * Implemented for cin in {64, 128, 256, 512, 1024} (the reference's list,
+ * dabnn/layers/BinConv.cpp:118; 1024 as two passes over 512 channels each, the
+ * second adding to the first) and cout % 8 == 0; other shapes return
+ * DAB_EUNSUPPORTED (use dab_fused_binarize_im2col + dab_bgemm, as the
  * reference's BGEMM arm does).
  */
 DAB_API int dab_bconv3x3(const uint64_t *x, int n, int h, int w, int cin, const uint64_t *wgt, int cout, int stride,
@@ -181,7 +183,7 @@ DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in
- * {64,128,256,512} takes the direct kernel (pack + bconv), anything else
+ * {64,128,256,512,1024} takes the direct kernel (pack + bconv), anything else
  * takes fused_binarize_im2col + bgemm on `wgt_t` (the transposed weights;
  * may be NULL when the direct kernel applies).
  * hwc_words = words per filter (weight.total()/weight.n).

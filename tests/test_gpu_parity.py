@@ -216,6 +216,10 @@ def test_im2col_transpose_bgemm_equals_baseline_bconv(dab):
     (6, 56, 56, 64, 64, 1, 1), (9, 28, 28, 128, 128, 1, 1), (17, 14, 14, 256, 256, 1, 1), (25, 7, 7, 512, 512, 1, 1),
     (10, 56, 56, 64, 128, 2, 1), (20, 28, 28, 128, 256, 2, 1), (30, 14, 14, 256, 512, 2, 1), (40, 9, 9, 64, 272, 1, 0), (48, 7, 7, 512, 512, 1, 1),
     (64, 56, 56, 64, 64, 1, 1), (200, 28, 28, 128, 128, 1, 1),
+    # 1024 input channels (dabnn/layers/BinConv.cpp:118 lists them): two passes over 512 channels each, the second
+    # adding to the first; a single tile, ragged tiles at stride 1 and 2, no padding, and enough work for the
+    # large-unit build
+    (1, 7, 7, 1024, 64, 1, 1), (3, 9, 11, 1024, 24, 2, 1), (2, 6, 6, 1024, 1024, 1, 0), (100, 7, 7, 1024, 1024, 1, 1),
 ])
 def test_bconv_3x3_matches_baseline_bconv(dab, n, h, w, cin, cout, stride, pad):
     cw = cin // 64
@@ -348,6 +352,13 @@ def test_bconv_3x3_unsupported_and_invalid(dab):
     x = torch.zeros((1, 4, 4, 1), dtype=torch.int64, device="cuda")
     with pytest.raises(DabUnsupported):  # cout not a multiple of 8
         dab.bconv_3x3(x, torch.zeros((5, 9), dtype=torch.int64, device="cuda"))
+    # 1024 input channels: counts only, no fused epilogue
+    x16 = torch.zeros((1, 4, 4, 16), dtype=torch.int64, device="cuda")
+    w16 = torch.zeros((8, 144), dtype=torch.int64, device="cuda")
+    ab = torch.zeros(8, device="cuda")
+    assert dab.bconv_3x3(x16, w16, 1, 1).shape == (1, 4, 4, 8)
+    with pytest.raises(DabUnsupported):
+        dab.bconv_3x3_affine_add(x16, w16, ab, ab, None, 1, 1)
     with pytest.raises(RuntimeError, match="smaller than the kernel"):
         dab.bconv_3x3(torch.zeros((1, 2, 2, 1), dtype=torch.int64, device="cuda"),
                       torch.zeros((8, 9), dtype=torch.int64, device="cuda"), 1, 0)
@@ -362,6 +373,7 @@ def test_bconv_3x3_unsupported_and_invalid(dab):
     (1, 6, 6, 256, 32, 1, 0, 1, 1),  # 1x1
     (1, 6, 6, 64, 12, 1, 0, 1, 1),  # 64 channels, not 3x3: unpadded filters against padded rows
     (1, 8, 8, 128, 20, 3, 1, 1, 1),  # cout not a multiple of 8 -> bgemm with a ragged last group
+    (2, 7, 7, 1024, 32, 3, 1, 1, 0),  # 1024 channels: direct, in two passes
 ])
 def test_binconv_layer_matches_reference_dispatch(dab, n, h, w, c, cout, k, pad, stride, method):
     x = rng(30).standard_normal((n, h, w, c)).astype(np.float32)

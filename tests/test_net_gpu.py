@@ -295,6 +295,41 @@ def test_bireal18_batch256_matches_cpu(mods, stem):
     n.close()
 
 
+def test_binconv_over_1024_channels_direct_equals_bgemm(mods):
+    """A binary convolution over 1024 channels takes the direct kernel (two passes over 512 channels each) when the net
+    optimizes and im2col + bgemm when it does not: the same blobs, and the CPU layers agree group by group; the Affine
+    behind it stays a layer of its own (no fused epilogue for this depth)."""
+    df, models, net = mods
+    r = np.random.default_rng(17)
+    w1 = (r.standard_normal((1024, 1, 1, 3)) / 2).astype(np.float32)
+    wf = r.standard_normal((64, 3, 3, 1024)).astype(np.float32)
+    a, b = (r.standard_normal(64) / 50).astype(np.float32), r.standard_normal(64).astype(np.float32)
+    inits = [{"name": "w1", "shape": [1024, 1, 1, 3], "data": w1, "align_hwc_to_128": False},
+             {"name": "w2", "shape": [64, 3, 3, 1024], "data": models.pack_weight(wf).ravel(), "align_hwc_to_128": True},
+             {"name": "a", "shape": [64], "data": a, "align_hwc_to_128": False},
+             {"name": "b", "shape": [64], "data": b, "align_hwc_to_128": False}]
+    layers = [{"type": "FpConv2D", "name": "conv", "input": "data", "weight": "w1", "output": "wide", "pads": [0] * 4,
+               "strides": [1, 1], "dilations": [1, 1]},
+              {"type": "BinConv2D", "name": "bconv", "input": "wide", "weight": "w2", "output": "cnt", "pads": [1] * 4,
+               "strides": [1, 1], "dilations": [1, 1]},
+              {"type": "Affine", "name": "affine", "input": "cnt", "a": "a", "b": "b", "output": "cnt_bn"}]
+    buf = df.write_model(layers, inits, [("data", [1, 9, 7, 3])])
+    batch = 3
+    x = r.standard_normal((batch, 9, 7, 3)).astype(np.float32)
+    outs = []
+    for optimize in (True, False):
+        n = net.Net(batch=batch, optimize=optimize).read_buf(buf)
+        descs = n.layers()
+        assert sum(("DIRECT_CONV" if optimize else "BGEMM") in d for d in descs) == 1
+        assert sum(d.startswith("Affine") for d in descs) == 1
+        n.run(x)
+        for i in range(batch):
+            assert check_every_segment(n, layers, inits, i) == 2  # the in-place Affine belongs to the BinConv group
+        outs.append(n.get_blob("cnt_bn").copy())
+        n.close()
+    np.testing.assert_array_equal(outs[0], outs[1])
+
+
 def test_stem_fusion_leaves_other_graphs_alone(mods):
     """The convolution + MaxPool pass needs the pool to be the only reader of the convolution's blob and a 3x3 stride-2
     pad-1 window: a second reader, or another window, keeps both layers, and every blob stays readable."""
