@@ -32,7 +32,7 @@ BATCH = 64
 # HBM traffic of the headline workload per kernel launch (bytes, mean of the seven shapes), measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --profile-mode` (summary: profiles/bconv3x3_config3_b64.md),
 # next to the algorithmic bytes (packed input + weights + fp32 output).
-TRAFFIC_BYTES_PER_LAUNCH = 26.44e6
+TRAFFIC_BYTES_PER_LAUNCH = 26.52e6
 ALGORITHMIC_BYTES_PER_LAUNCH = 21.10e6
 
 
