@@ -3,15 +3,17 @@
 // per depth group, fp32 accuracy), with the optional Affine and Relu of dab_fconv_affine_relu in the same pass.
 //
 // A depth group of the matrix instruction (32 depths) is one tap's 32 channels, so there is no im2col stage and no
-// pixel tile in LDS: a wave owns 64 output pixels (four tiles of 16 along an image row) and all output channels, and
-// for every tap a lane fetches the eight channels 8 * (lane / 16) .. + 7 of its pixel of each tile straight from the
-// image -- 16 lanes x 4 groups read 16 pixels x 128 contiguous bytes -- and splits them in registers.  Out-of-image taps
-// read zero through the buffer descriptor.  The filters are split once per block into three planes of bf16 in LDS
-// ([plane][output channel][tap][32] with eight elements of padding per channel: a quarter wave's 16-byte reads hit
-// all banks); a filter fragment (16 channels x 32 depths of one tap) is read once per tap and used for the wave's four
-// pixel tiles.  The output channels are the rows of the matrix instruction and the pixels its columns, so a lane ends
-// up with four consecutive channels of one pixel: one 16-byte store.  Waves are independent (no barrier after the
-// filters are in place) and persistent over their share of the 64-pixel items.
+// pixel tile in LDS: a wave owns a column of four 16-pixel tiles (four consecutive output rows at one x tile) and all
+// output channels.  For every horizontal tap a lane fetches the eight channels 8 * (lane / 16) .. + 7 of its pixel in
+// each of the six input rows under the column straight from the image -- 16 lanes x 4 groups read 16 pixels x 128
+// contiguous bytes -- and splits them in registers; a split row serves the three output rows it is a vertical tap of.
+// Out-of-image taps read zero through the buffer descriptor.  The next tap's rows are in flight while this one's
+// products are made.  The filters are split once per block into three planes of bf16 in LDS ([plane][output
+// channel][tap][32] with eight elements of padding per channel: a quarter wave's 16-byte reads hit all banks); a
+// filter fragment (16 channels x 32 depths of one tap) is read once per tap and used for the wave's four tiles.  The
+// output channels are the rows of the matrix instruction and the pixels its columns, so a lane ends up with four
+// consecutive channels of one pixel: one 16-byte store.  Waves are independent (no barrier after the filters are in
+// place) and persistent over their share of the items.
 #include <cfloat>
 #include <type_traits>
 
@@ -25,9 +27,9 @@ struct FconvC32Args {
     int relu;
     int h, wd, oh, ow, cout, pad_h, pad_w;
     uint32_t x_bytes;
-    int tiles;          // 16-pixel tiles of the output: n * oh * ow / 16
-    int items;          // groups of four tiles
-    FastDiv div_tiles_per_row, div_oh;
+    int items;          // columns of four tiles: n * ceil(oh / 4) * (ow / 16)
+    int row_groups;     // ceil(oh / 4)
+    FastDiv div_tiles_per_row, div_row_groups;
     int tiles_per_row;
 };
 
@@ -67,105 +69,67 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
 
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, p.x_bytes);
     typedef float f32x4r __attribute__((ext_vector_type(4)));
+    typedef SplitFrag8::u4 u4;
     // A block works through a contiguous range of items, its waves side by side: the image rows above and below the
     // ones it is on were fetched by the block itself a moment ago and are still in its L2 (with the items dealt to all
     // waves in turn every row was fetched from memory twice, by blocks on different XCDs).
     const int per = p.items / (int)gridDim.x, extra = p.items - per * (int)gridDim.x, b = (int)blockIdx.x;
     const int first = b * per + (b < extra ? b : extra), last = first + per + (b < extra ? 1 : 0);
 
-    for (int item = first + wave; item < last; item += kC32Threads / 64) {
-        // the lane's pixel of each tile: byte offset of its window's first tap (may lie outside the image: then the
-        // row or column test below sends the load out of range), and its coordinates for those tests
-        int off0[PT], iy0[PT], ix0[PT];
-#pragma unroll
-        for (int t = 0; t < PT; ++t) {
-            const int T = item * PT + t;
-            const uint32_t row = p.div_tiles_per_row.div((uint32_t)T);
-            const int xt = T - (int)row * p.tiles_per_row;
-            const uint32_t img = p.div_oh.div(row);
-            const int oy = (int)(row - img * (uint32_t)p.oh);
-            const bool tile_ok = T < p.tiles;
-            iy0[t] = tile_ok ? oy - p.pad_h : -0x40000000;  // a tile past the end reads nothing
-            ix0[t] = xt * 16 + f_i - p.pad_w;
-            off0[t] = tile_ok ? (((int)img * p.h + iy0[t]) * p.wd + ix0[t]) * 128 + g * 32 : 0;
-        }
-        auto fetch = [&](int tap, f32x4r (&lo)[PT], f32x4r (&hi)[PT]) {
-            const int ty = tap / KW, tx = tap - ty * KW;
-#pragma unroll
-            for (int t = 0; t < PT; ++t) {
-                const bool ok = (unsigned)(iy0[t] + ty) < (unsigned)p.h && (unsigned)(ix0[t] + tx) < (unsigned)p.wd;
-                const uint32_t off = ok ? (uint32_t)(off0[t] + (ty * p.wd + tx) * 128) : kC32Oob;
-                lo[t] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0));
-                hi[t] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(off + 16u), 0, 0));
-            }
-        };
-        // a filter fragment: output channels 16 * nt + f_i, depths 8 * g .. + 7 of the tap
-        auto filter_frag = [&](auto filters_special, int nt, int tap) {
-            const uint16_t *src = planes + (nt * 16 + f_i) * ROW + tap * 32 + 8 * g;
-            SplitFrag8 f;
-            f.hi = *reinterpret_cast<const SplitFrag8::u4 *>(src);
-            f.mid = *reinterpret_cast<const SplitFrag8::u4 *>(src + PLANE);
-            f.lo = *reinterpret_cast<const SplitFrag8::u4 *>(src + 2 * PLANE);
-            f.hif = f.hi;
-            if constexpr (decltype(filters_special)::value) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
-            }
-            return f;
-        };
-
-        f32x4w acc[PT][NT];
-#pragma unroll
-        for (int t = 0; t < PT; ++t)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) acc[t][nt] = f32x4w{0.f, 0.f, 0.f, 0.f};
-
-        f32x4r raw_lo[PT], raw_hi[PT];
-        fetch(0, raw_lo, raw_hi);
-        auto all_taps = [&](auto filters_special) {
-        // the taps one after the other (not unrolled: the compiler would otherwise start all nine taps' loads at once
-        // and spill); the next tap's pixels are on their way while this tap is multiplied
-#pragma unroll 1
-        for (int tap = 0; tap < TAPS; ++tap) {
-            SplitFrag8 px[PT];
-            uint32_t magnitude = 0;
-#pragma unroll
-            for (int t = 0; t < PT; ++t) {
-                const float v[8] = {raw_lo[t][0], raw_lo[t][1], raw_lo[t][2], raw_lo[t][3],
-                                    raw_hi[t][0], raw_hi[t][1], raw_hi[t][2], raw_hi[t][3]};
-                magnitude = px[t].set_finite(v, magnitude);
-            }
-            if (__builtin_amdgcn_ballot_w64(!bf16_pairs_finite(magnitude)) != 0) {
-                // an infinity or a NaN among the wave's pixels of this tap: the split that keeps it out of the cross terms
-#pragma unroll
-                for (int t = 0; t < PT; ++t) {
-                    const float v[8] = {raw_lo[t][0], raw_lo[t][1], raw_lo[t][2], raw_lo[t][3],
-                                        raw_hi[t][0], raw_hi[t][1], raw_hi[t][2], raw_hi[t][3]};
-                    px[t].set(v);
-                }
-            }
-            if (tap + 1 < TAPS) fetch(tap + 1, raw_lo, raw_hi);
-            // rows of the product = output channels (the filter fragment), columns = pixels
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const SplitFrag8 f = filter_frag(filters_special, nt, tap);
-                mfma6_16x16x32(acc[0][nt], acc[1][nt], f, px[0], px[1]);
-                mfma6_16x16x32(acc[2][nt], acc[3][nt], f, px[2], px[3]);
-            }
-        }
-        };
-        if (w_special)
-            all_taps(std::true_type{});
-        else
-            all_taps(std::false_type{});
-
-        // accumulator element e of lane l: output channel 16 * nt + 4 * (l / 16) + e of pixel l % 16
-        auto store_all = [&]() {
+    // An item is a column of four tiles: output rows oy0 .. oy0 + 3 of one image at the 16 pixels of one x tile.  An
+    // input row's pixels at horizontal tap tx then serve three of the item's output rows (vertical taps 0, 1, 2), so a
+    // fetched and split fragment is used for three tiles' products: KH + 3 fragments per horizontal tap instead of
+    // 4 * KH -- the splitting, which bounds the kernel with few output channels, is halved.
+    constexpr int ROWS = PT + KH - 1;
+    struct Place {
+        int img, oy0, xt;
+        int off0;  // byte offset of this lane's eight channels at input row oy0 - pad, column of tap 0 (may lie outside the image)
+    };
+    auto locate = [&](int item) {
+        Place q;
+        const uint32_t rowg = p.div_tiles_per_row.div((uint32_t)item);
+        q.xt = item - (int)rowg * p.tiles_per_row;
+        q.img = (int)p.div_row_groups.div(rowg);
+        q.oy0 = ((int)rowg - q.img * p.row_groups) * PT;
+        q.off0 = ((q.img * p.h + q.oy0 - p.pad_h) * p.wd + q.xt * 16 + f_i - p.pad_w) * 128 + g * 32;
+        return q;
+    };
+    // the eight channels of this lane's pixel at input row (oy0 - pad + j), horizontal tap tx; zero outside the image
+    // and for an item beyond the block's range
+    auto fetch = [&](const Place &q, bool item_ok, int j, int tx, f32x4r (&r)[2]) __attribute__((always_inline)) {
+        const bool ok = item_ok && (unsigned)(q.xt * 16 + f_i - p.pad_w + tx) < (unsigned)p.wd && (unsigned)(q.oy0 - p.pad_h + j) < (unsigned)p.h;
+        const uint32_t off = ok ? (uint32_t)(q.off0 + (j * p.wd + tx) * 128) : kC32Oob;
+        r[0] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0));
+        r[1] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(off + 16u), 0, 0));
+    };
+    auto filter_at = [&](int nt, int ty, int tx) { return planes + (nt * 16 + f_i) * ROW + (ty * KW + tx) * 32 + 8 * g; };
+    // accumulator element e of lane l: output channel 16 * nt + 4 * (l / 16) + e of pixel l % 16
+    auto finish = [&](float v, float bias, float fa, float fb) {
 #pragma clang fp contract(off)
+        if (p.bias) v = v + bias;
+        if (p.aff_a) {
+            const float prod = fa * v;
+            v = prod + fb;
+        }
+        if (p.relu) v = v < 0.f ? 0.f : v;  // std::max(v, 0.f): a NaN stays
+        return v;
+    };
+
+    Place here = locate(first + wave);
+    f32x4r raw[ROWS][2];  // the six input rows of the next horizontal tap, in flight while this one's products are made
+#pragma unroll
+    for (int j = 0; j < ROWS; ++j) fetch(here, first + wave < last, j, 0, raw[j]);
+
+    f32x4w acc[PT][NT];
+    // Writes the item at `at`, whose sums are in acc (special: an infinity or a NaN among its pixels or in the filters).
+    auto write_item = [&](const Place &at, bool special) __attribute__((always_inline)) {
+        int g_now = g;
+        asm volatile("" : "+v"(g_now));  // what follows is read per item: hoisted out of the item loop it would be spilled
+        if (!special) {
             float bs[NT][4], as[NT][4], bb[NT][4];
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
-                const int co = nt * 16 + 4 * g;
+                const int co = nt * 16 + 4 * g_now;
                 const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
                 const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
                 const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -177,28 +141,118 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
             // still in the write path
 #pragma unroll
             for (int t = 0; t < PT; ++t) {
-                const int T = item * PT + t;
-                if (T >= p.tiles) continue;
+                if (at.oy0 + t >= p.oh) continue;
+                const size_t m = ((size_t)at.img * p.oh + at.oy0 + t) * p.ow + at.xt * 16 + f_i;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     float v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = acc[t][nt][e];
-                        if (p.bias) v[e] = v[e] + bs[nt][e];
-                        if (p.aff_a) {
-                            const float prod = as[nt][e] * v[e];
-                            v[e] = prod + bb[nt][e];
-                        }
-                        if (p.relu) v[e] = v[e] < 0.f ? 0.f : v[e];  // std::max(v, 0.f): a NaN stays
-                    }
-                    *reinterpret_cast<float4 *>(p.out + ((size_t)T * 16 + f_i) * COUT + nt * 16 + 4 * g) =
-                        make_float4(v[0], v[1], v[2], v[3]);
+                    for (int e = 0; e < 4; ++e) v[e] = finish(acc[t][nt][e], bs[nt][e], as[nt][e], bb[nt][e]);
+                    *reinterpret_cast<float4 *>(p.out + m * COUT + 4 * g_now + nt * 16) = make_float4(v[0], v[1], v[2], v[3]);
                 }
             }
-        };
-        store_all();
+        } else {
+            // The item is made again, one tile and one tap at a time, with the split that keeps an infinity or a NaN
+            // whole in hi and takes copies with the non-finite values zeroed for the cross terms (Inf * 0 would make a
+            // NaN of a sum that is an infinity).
+#pragma unroll 1
+            for (int t = 0; t < PT; ++t) {
+                if (at.oy0 + t >= p.oh) break;
+                const size_t m = ((size_t)at.img * p.oh + at.oy0 + t) * p.ow + at.xt * 16 + f_i;
+#pragma unroll 1
+                for (int nt = 0; nt < NT; ++nt) {
+                    f32x4w one = f32x4w{0.f, 0.f, 0.f, 0.f}, none = one;
+#pragma unroll 1
+                    for (int tap = 0; tap < TAPS; ++tap) {
+                        const int ty = tap / KW, tx = tap - ty * KW;
+                        f32x4r r[2];
+                        fetch(at, true, t + ty, tx, r);
+                        const float v[8] = {r[0][0], r[0][1], r[0][2], r[0][3], r[1][0], r[1][1], r[1][2], r[1][3]};
+                        SplitFrag8 px, f;
+                        px.set(v);
+                        const uint16_t *src = filter_at(nt, ty, tx);
+                        f.hi = *reinterpret_cast<const u4 *>(src), f.mid = *reinterpret_cast<const u4 *>(src + PLANE);
+                        f.lo = *reinterpret_cast<const u4 *>(src + 2 * PLANE);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
+                        mfma6_16x16x32(one, none, f, px, px);
+                    }
+                    const int co = nt * 16 + 4 * g_now;
+                    const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    *reinterpret_cast<float4 *>(p.out + m * COUT + co) =
+                        make_float4(finish(one[0], bias.x, fa.x, fb.x), finish(one[1], bias.y, fa.y, fb.y),
+                                    finish(one[2], bias.z, fa.z, fb.z), finish(one[3], bias.w, fa.w, fb.w));
+                }
+            }
+        }
+    };
+
+    // An item's results are written after the first split of the next item, just before a long run of products: the
+    // wait for the next fetched rows also waits for every store before it to be acknowledged (one counter covers
+    // both, and loads and stores complete in no fixed order), which by then has long happened.
+    Place done = here;
+    bool have_done = false, done_special = false;
+    for (int item = first + wave; item < last; item += kC32Threads / 64) {
+        const Place next = locate(item + kC32Threads / 64);
+        const bool next_ok = item + kC32Threads / 64 < last;
+        uint32_t magnitude = 0;
+
+#pragma unroll 1
+        for (int tx = 0; tx < KW; ++tx) {
+            u4 hi[ROWS], mid[ROWS], lo[ROWS];
+#pragma unroll
+            for (int j = 0; j < ROWS; ++j) {
+                const float v[8] = {raw[j][0][0], raw[j][0][1], raw[j][0][2], raw[j][0][3], raw[j][1][0], raw[j][1][1], raw[j][1][2], raw[j][1][3]};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const SplitPair sp = split_pair_finite(v[2 * e], v[2 * e + 1]);
+                    hi[j][e] = sp.hi, mid[j][e] = sp.mid, lo[j][e] = sp.lo;
+                    magnitude = bf16_pair_max(magnitude, sp.hi);
+                }
+            }
+            // the next tap's rows, or the next item's first
+            if (tx + 1 < KW) {
+#pragma unroll
+                for (int j = 0; j < ROWS; ++j) fetch(here, true, j, tx + 1, raw[j]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < ROWS; ++j) fetch(next, next_ok, j, 0, raw[j]);
+            }
+            if (tx == 0) {
+                if (have_done) write_item(done, done_special);
+#pragma unroll
+                for (int t = 0; t < PT; ++t)
+#pragma unroll
+                    for (int nt = 0; nt < NT; ++nt) acc[t][nt] = f32x4w{0.f, 0.f, 0.f, 0.f};
+            }
+            // rows of the product = output channels (the filter fragment), columns = pixels; output row t takes input
+            // row t + ty
+            auto frag = [](const u4 &h, const u4 &m, const u4 &l) {
+                SplitFrag8 f;
+                f.hi = h, f.hif = h, f.mid = m, f.lo = l;
+                return f;
+            };
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+                for (int ty = 0; ty < KH; ++ty) {
+                    const uint16_t *src = filter_at(nt, ty, tx);
+                    const SplitFrag8 f = frag(*reinterpret_cast<const u4 *>(src), *reinterpret_cast<const u4 *>(src + PLANE),
+                                              *reinterpret_cast<const u4 *>(src + 2 * PLANE));
+                    mfma6_16x16x32(acc[0][nt], acc[1][nt], f, frag(hi[ty], mid[ty], lo[ty]), frag(hi[ty + 1], mid[ty + 1], lo[ty + 1]));
+                    mfma6_16x16x32(acc[2][nt], acc[3][nt], f, frag(hi[ty + 2], mid[ty + 2], lo[ty + 2]),
+                                   frag(hi[ty + 3], mid[ty + 3], lo[ty + 3]));
+                    __builtin_amdgcn_sched_barrier(0);  // filter fragments are read as they are needed, not all up front
+                }
+            }
+        }
+        done = here, have_done = true;
+        done_special = w_special || __builtin_amdgcn_ballot_w64(!bf16_pairs_finite(magnitude)) != 0;
+        here = next;
     }
+    if (have_done) write_item(done, done_special);
 }
 
 // Whether the shapes are this kernel's and the problem is large enough to fill its persistent waves (buffer alignment
@@ -211,7 +265,7 @@ bool fconv_c32_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int 
     if (in_bytes >= (1ll << 31) || tiles >= (1ll << 30)) return false;
     const long long waves = (long long)(simd_count() / 4) * (kC32Threads / 64);
     // smaller problems: the general kernel's tiles fill the chip better
-    return (tiles + kC32PixelTiles - 1) / kC32PixelTiles >= 2 * waves;
+    return (long long)n * ((oh + kC32PixelTiles - 1) / kC32PixelTiles) * (ow / 16) >= 2 * waves;
 }
 
 // Runs the convolution if fconv_c32_takes says so and the buffers are 16-byte aligned; returns 1 when it did, 0 when
@@ -224,15 +278,14 @@ int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, 
     if (bias) align |= reinterpret_cast<uintptr_t>(bias);
     if (aff_a) align |= reinterpret_cast<uintptr_t>(aff_a) | reinterpret_cast<uintptr_t>(aff_b);
     if (align % 16 != 0) return 0;
-    const long long tiles = (long long)n * oh * ow / 16;
     const int blocks = simd_count() / 4;  // one block of eight waves per CU (the filter planes take most of its LDS)
     FconvC32Args a;
     a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.out = out, a.relu = relu;
     a.h = h, a.wd = w, a.oh = oh, a.ow = ow, a.cout = cout, a.pad_h = pad_h, a.pad_w = pad_w;
     a.x_bytes = (uint32_t)((long long)n * h * w * 128);
-    a.tiles = (int)tiles, a.items = (int)((tiles + kC32PixelTiles - 1) / kC32PixelTiles);
-    a.tiles_per_row = ow / 16;
-    a.div_tiles_per_row = FastDiv((uint32_t)a.tiles_per_row), a.div_oh = FastDiv((uint32_t)oh);
+    a.row_groups = (oh + kC32PixelTiles - 1) / kC32PixelTiles, a.tiles_per_row = ow / 16;
+    a.items = n * a.row_groups * a.tiles_per_row;
+    a.div_tiles_per_row = FastDiv((uint32_t)a.tiles_per_row), a.div_row_groups = FastDiv((uint32_t)a.row_groups);
     if (cout == 32)
         hipLaunchKernelGGL((fconv_c32_kernel<2, 3, 3>), dim3(blocks), dim3(kC32Threads), 0, s, a);
     else
