@@ -4,16 +4,17 @@
 //
 // A depth group of the matrix instruction (32 depths) is one tap's 32 channels, so there is no im2col stage and no
 // pixel tile in LDS: a wave owns a column of four 16-pixel tiles (four consecutive output rows at one x tile) and all
-// output channels.  For every horizontal tap a lane fetches the eight channels 8 * (lane / 16) .. + 7 of its pixel in
-// each of the six input rows under the column straight from the image -- 16 lanes x 4 groups read 16 pixels x 128
-// contiguous bytes -- and splits them in registers; a split row serves the three output rows it is a vertical tap of.
-// Out-of-image taps read zero through the buffer descriptor.  The next tap's rows are in flight while this one's
-// products are made.  The filters are split once per block into three planes of bf16 in LDS ([plane][output
-// channel][tap][32] with eight elements of padding per channel: a quarter wave's 16-byte reads hit all banks); a
-// filter fragment (16 channels x 32 depths of one tap) is read once per tap and used for the wave's four tiles.  The
-// output channels are the rows of the matrix instruction and the pixels its columns, so a lane ends up with four
-// consecutive channels of one pixel: one 16-byte store.  Waves are independent (no barrier after the filters are in
-// place) and persistent over their share of the items.
+// output channels.  A lane fetches the eight channels 8 * (lane / 16) .. + 7 of its pixel in each of the six input
+// rows under the column straight from the image -- 16 lanes x 4 groups read 16 pixels x 128 contiguous bytes -- and
+// splits them in registers, once: a split row serves the three output rows it is a vertical tap of, and the three
+// horizontal taps are the same values one lane over (lane-shifting moves, with the two pixels beside the tile fetched
+// and split as a seventh row).  Out-of-image taps read zero through the buffer descriptor.  The next item's rows are
+// in flight while this one's last products are made.  The filters are split once per block into three planes of bf16
+// in LDS ([plane][output channel][tap][32] with eight elements of padding per channel: a quarter wave's 16-byte reads
+// hit all banks); a filter fragment (16 channels x 32 depths of one tap) is read once per tap and used for the wave's
+// four tiles.  The output channels are the rows of the matrix instruction and the pixels its columns, so a lane ends
+// up with four consecutive channels of one pixel: one 16-byte store.  Waves are independent (no barrier after the
+// filters are in place) and take their items from a counter of the block.
 #include <cfloat>
 #include <type_traits>
 
@@ -43,11 +44,29 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     constexpr int PLANE = COUT * ROW;      // elements per plane (hi, mid, lo)
     __shared__ __attribute__((aligned(16))) uint16_t planes[3 * PLANE];
     __shared__ int filter_special;  // a filter value is an infinity or a NaN
+    __shared__ int next_item;       // the first item of the block's range that no wave has taken
+    // bias, Affine a and b per output channel (zeros where the layer has none): read from here when an item is written,
+    // so that no load is outstanding among the stores -- loads and stores share one counter and complete in no fixed
+    // order, and a wait for such a load would also wait for every store before it to be acknowledged
+    __shared__ __attribute__((aligned(16))) float per_channel[3][COUT];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int g = lane >> 4, f_i = lane & 15;
 
-    if (tid == 0) filter_special = 0;
+    // A block works through a contiguous range of items, its waves side by side: the image rows above and below the
+    // ones it is on were fetched by the block itself a moment ago and are still in its L2 (with the items dealt to all
+    // waves in turn every row was fetched from memory twice, by blocks on different XCDs).  A wave takes its next item
+    // from a counter: of the two waves of a SIMD the older one is served first and gets through its items faster, and
+    // with equal shares the other would finish its last quarter alone, its vector and matrix instructions no longer
+    // overlapping with anyone's.
+    const int per = p.items / (int)gridDim.x, extra = p.items - per * (int)gridDim.x, b = (int)blockIdx.x;
+    const int first = b * per + (b < extra ? b : extra), last = first + per + (b < extra ? 1 : 0);
+    if (tid == 0) filter_special = 0, next_item = first + kC32Threads / 64;
+    if (tid < COUT) {
+        per_channel[0][tid] = p.bias ? p.bias[tid] : 0.f;
+        per_channel[1][tid] = p.aff_a ? p.aff_a[tid] : 0.f;
+        per_channel[2][tid] = p.aff_a ? p.aff_b[tid] : 0.f;
+    }
     __syncthreads();
     {
         bool special = false;
@@ -70,12 +89,6 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     const __amdgpu_buffer_rsrc_t x_rsrc = make_rsrc(p.x, p.x_bytes);
     typedef float f32x4r __attribute__((ext_vector_type(4)));
     typedef SplitFrag8::u4 u4;
-    // A block works through a contiguous range of items, its waves side by side: the image rows above and below the
-    // ones it is on were fetched by the block itself a moment ago and are still in its L2 (with the items dealt to all
-    // waves in turn every row was fetched from memory twice, by blocks on different XCDs).
-    const int per = p.items / (int)gridDim.x, extra = p.items - per * (int)gridDim.x, b = (int)blockIdx.x;
-    const int first = b * per + (b < extra ? b : extra), last = first + per + (b < extra ? 1 : 0);
-
     // An item is a column of four tiles: output rows oy0 .. oy0 + 3 of one image at the 16 pixels of one x tile.  An
     // input row's pixels at horizontal tap tx then serve three of the item's output rows (vertical taps 0, 1, 2), so a
     // fetched and split fragment is used for three tiles' products: KH + 3 fragments per horizontal tap instead of
@@ -115,10 +128,23 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
         return v;
     };
 
+    static_assert(KW == 3, "the horizontal taps are the fetched pixels and their two neighbours");
+    // The halo of an item: lane l % 16 = j < 6 fetches the pixel left of the item's 16 (horizontal tap 0 of the first
+    // pixel) in input row j, lane l % 16 = 8 + j the pixel right of them (tap 2 of the last).
+    auto fetch_halo = [&](const Place &q, bool item_ok, f32x4r (&r)[2]) __attribute__((always_inline)) {
+        const int j = f_i & 7, col = q.xt * 16 - p.pad_w + (f_i >> 3) * 17;
+        const bool ok = item_ok && j < ROWS && (unsigned)col < (unsigned)p.wd && (unsigned)(q.oy0 - p.pad_h + j) < (unsigned)p.h;
+        const uint32_t off = ok ? (uint32_t)(q.off0 + (j * p.wd + (f_i >> 3) * 17 - f_i) * 128) : kC32Oob;
+        r[0] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)off, 0, 0));
+        r[1] = __builtin_bit_cast(f32x4r, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, (int)(off + 16u), 0, 0));
+    };
     Place here = locate(first + wave);
-    f32x4r raw[ROWS][2];  // the six input rows of the next horizontal tap, in flight while this one's products are made
+    // the next item's six input rows (the pixels of horizontal tap 1) and halo, in flight while this one's last
+    // products are made
+    f32x4r raw[ROWS][2], raw_halo[2];
 #pragma unroll
-    for (int j = 0; j < ROWS; ++j) fetch(here, first + wave < last, j, 0, raw[j]);
+    for (int j = 0; j < ROWS; ++j) fetch(here, first + wave < last, j, 1, raw[j]);
+    fetch_halo(here, first + wave < last, raw_halo);
 
     f32x4w acc[PT][NT];
     // Writes the item at `at`, whose sums are in acc (special: an infinity or a NaN among its pixels or in the filters).
@@ -130,9 +156,9 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const int co = nt * 16 + 4 * g_now;
-                const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-                const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-                const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 bias = *reinterpret_cast<const float4 *>(per_channel[0] + co);
+                const float4 fa = *reinterpret_cast<const float4 *>(per_channel[1] + co);
+                const float4 fb = *reinterpret_cast<const float4 *>(per_channel[2] + co);
                 bs[nt][0] = bias.x, bs[nt][1] = bias.y, bs[nt][2] = bias.z, bs[nt][3] = bias.w;
                 as[nt][0] = fa.x, as[nt][1] = fa.y, as[nt][2] = fa.z, as[nt][3] = fa.w;
                 bb[nt][0] = fb.x, bb[nt][1] = fb.y, bb[nt][2] = fb.z, bb[nt][3] = fb.w;
@@ -178,9 +204,9 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                         mfma6_16x16x32(one, none, f, px, px);
                     }
                     const int co = nt * 16 + 4 * g_now;
-                    const float4 bias = p.bias ? *reinterpret_cast<const float4 *>(p.bias + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-                    const float4 fa = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_a + co) : make_float4(0.f, 0.f, 0.f, 0.f);
-                    const float4 fb = p.aff_a ? *reinterpret_cast<const float4 *>(p.aff_b + co) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float4 bias = *reinterpret_cast<const float4 *>(per_channel[0] + co);
+                    const float4 fa = *reinterpret_cast<const float4 *>(per_channel[1] + co);
+                    const float4 fb = *reinterpret_cast<const float4 *>(per_channel[2] + co);
                     *reinterpret_cast<float4 *>(p.out + m * COUT + co) =
                         make_float4(finish(one[0], bias.x, fa.x, fb.x), finish(one[1], bias.y, fa.y, fb.y),
                                     finish(one[2], bias.z, fa.z, fb.z), finish(one[3], bias.w, fa.w, fb.w));
@@ -189,68 +215,114 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
         }
     };
 
-    // An item's results are written after the first split of the next item, just before a long run of products: the
-    // wait for the next fetched rows also waits for every store before it to be acknowledged (one counter covers
-    // both, and loads and stores complete in no fixed order), which by then has long happened.
+    // An item's results are written after the split of the next item, just before a long run of products: the wait
+    // for the next fetched rows also waits for every store before it to be acknowledged (one counter covers both, and
+    // loads and stores complete in no fixed order), which by then has long happened.
     Place done = here;
     bool have_done = false, done_special = false;
-    for (int item = first + wave; item < last; item += kC32Threads / 64) {
-        const Place next = locate(item + kC32Threads / 64);
-        const bool next_ok = item + kC32Threads / 64 < last;
-        uint32_t magnitude = 0;
-
-#pragma unroll 1
-        for (int tx = 0; tx < KW; ++tx) {
-            u4 hi[ROWS], mid[ROWS], lo[ROWS];
+    struct Row {
+        u4 hi, mid, lo;
+    };
+    auto split_row = [&](const f32x4r (&r)[2], uint32_t &magnitude) __attribute__((always_inline)) {
+        const float v[8] = {r[0][0], r[0][1], r[0][2], r[0][3], r[1][0], r[1][1], r[1][2], r[1][3]};
+        Row out;
 #pragma unroll
-            for (int j = 0; j < ROWS; ++j) {
-                const float v[8] = {raw[j][0][0], raw[j][0][1], raw[j][0][2], raw[j][0][3], raw[j][1][0], raw[j][1][1], raw[j][1][2], raw[j][1][3]};
+        for (int e = 0; e < 4; ++e) {
+            const SplitPair sp = split_pair_finite(v[2 * e], v[2 * e + 1]);
+            out.hi[e] = sp.hi, out.mid[e] = sp.mid, out.lo[e] = sp.lo;
+            magnitude = bf16_pair_max(magnitude, sp.hi);
+        }
+        return out;
+    };
+    for (int item = first + wave; item < last;) {
+        int taken = 0;
+        if (lane == 0) taken = atomicAdd(&next_item, 1);
+        const int next_index = __builtin_amdgcn_readfirstlane(taken);
+        const Place next = locate(next_index);
+        const bool next_ok = next_index < last;
+        uint32_t magnitude = 0;
+        // Every pixel is fetched and split once: the pixels of horizontal tap 1, and the halo.  Taps 0 and 2 are the
+        // same values one lane over (a lane's neighbours in its group of 16 hold the neighbouring pixels' same eight
+        // channels), moved with the lane-shifting form of v_mov; the end lane takes its value from the halo row.
+        Row centre[ROWS];
+#pragma unroll
+        for (int j = 0; j < ROWS; ++j) centre[j] = split_row(raw[j], magnitude);
+        const Row halo = split_row(raw_halo, magnitude);
+
+        if (have_done) write_item(done, done_special);
+#pragma unroll
+        for (int t = 0; t < PT; ++t)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) acc[t][nt] = f32x4w{0.f, 0.f, 0.f, 0.f};
+
+        // input row j as horizontal tap TX sees it
+        auto shifted = [&](auto tx_c, auto j_c) __attribute__((always_inline)) {
+            constexpr int TX = decltype(tx_c)::value, J = decltype(j_c)::value;
+            if constexpr (TX == 1) {
+                return centre[J];
+            } else {
+                Row out;
+                auto move = [&](uint32_t c, uint32_t h) {
+                    // row_shl:n (0x100 + n): lane i takes lane i + n's; row_shr:n (0x110 + n): lane i - n's; a lane
+                    // without a source keeps the first argument
+                    if constexpr (TX == 0) {
+                        const int end = J == 0 ? (int)h : __builtin_amdgcn_update_dpp(0, (int)h, 0x100 + (J == 0 ? 1 : J), 0xf, 0xf, true);
+                        return (uint32_t)__builtin_amdgcn_update_dpp(end, (int)c, 0x111, 0xf, 0xf, false);
+                    } else {
+                        const int end = __builtin_amdgcn_update_dpp(0, (int)h, 0x110 + (7 - J), 0xf, 0xf, true);
+                        return (uint32_t)__builtin_amdgcn_update_dpp(end, (int)c, 0x101, 0xf, 0xf, false);
+                    }
+                };
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const SplitPair sp = split_pair_finite(v[2 * e], v[2 * e + 1]);
-                    hi[j][e] = sp.hi, mid[j][e] = sp.mid, lo[j][e] = sp.lo;
-                    magnitude = bf16_pair_max(magnitude, sp.hi);
+                    out.hi[e] = move(centre[J].hi[e], halo.hi[e]);
+                    out.mid[e] = move(centre[J].mid[e], halo.mid[e]);
+                    out.lo[e] = move(centre[J].lo[e], halo.lo[e]);
                 }
+                return out;
             }
-            // the next tap's rows, or the next item's first
-            if (tx + 1 < KW) {
+        };
+        auto frag = [](const u4 &h, const u4 &m, const u4 &l) {
+            SplitFrag8 f;
+            f.hi = h, f.hif = h, f.mid = m, f.lo = l;
+            return f;
+        };
+        auto of_row = [&](const Row &r) { return frag(r.hi, r.mid, r.lo); };
+        // rows of the product = output channels (the filter fragment), columns = pixels; output row t takes input row
+        // t + ty.  The rows of a tap are made as the vertical taps first need them: four, then one, then one.
+        auto phase = [&](auto tx_c, auto &&after_first) __attribute__((always_inline)) {
+            constexpr int TX = decltype(tx_c)::value;
+            Row r0 = shifted(tx_c, std::integral_constant<int, 0>{}), r1 = shifted(tx_c, std::integral_constant<int, 1>{});
+            Row r2 = shifted(tx_c, std::integral_constant<int, 2>{}), r3 = shifted(tx_c, std::integral_constant<int, 3>{});
+            auto products = [&](int ty, const Row &a, const Row &b, const Row &c, const Row &d) __attribute__((always_inline)) {
 #pragma unroll
-                for (int j = 0; j < ROWS; ++j) fetch(here, true, j, tx + 1, raw[j]);
-            } else {
-#pragma unroll
-                for (int j = 0; j < ROWS; ++j) fetch(next, next_ok, j, 0, raw[j]);
-            }
-            if (tx == 0) {
-                if (have_done) write_item(done, done_special);
-#pragma unroll
-                for (int t = 0; t < PT; ++t)
-#pragma unroll
-                    for (int nt = 0; nt < NT; ++nt) acc[t][nt] = f32x4w{0.f, 0.f, 0.f, 0.f};
-            }
-            // rows of the product = output channels (the filter fragment), columns = pixels; output row t takes input
-            // row t + ty
-            auto frag = [](const u4 &h, const u4 &m, const u4 &l) {
-                SplitFrag8 f;
-                f.hi = h, f.hif = h, f.mid = m, f.lo = l;
-                return f;
-            };
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-                for (int ty = 0; ty < KH; ++ty) {
-                    const uint16_t *src = filter_at(nt, ty, tx);
+                for (int nt = 0; nt < NT; ++nt) {
+                    const uint16_t *src = filter_at(nt, ty, TX);
                     const SplitFrag8 f = frag(*reinterpret_cast<const u4 *>(src), *reinterpret_cast<const u4 *>(src + PLANE),
                                               *reinterpret_cast<const u4 *>(src + 2 * PLANE));
-                    mfma6_16x16x32(acc[0][nt], acc[1][nt], f, frag(hi[ty], mid[ty], lo[ty]), frag(hi[ty + 1], mid[ty + 1], lo[ty + 1]));
-                    mfma6_16x16x32(acc[2][nt], acc[3][nt], f, frag(hi[ty + 2], mid[ty + 2], lo[ty + 2]),
-                                   frag(hi[ty + 3], mid[ty + 3], lo[ty + 3]));
-                    __builtin_amdgcn_sched_barrier(0);  // filter fragments are read as they are needed, not all up front
+                    mfma6_16x16x32(acc[0][nt], acc[1][nt], f, of_row(a), of_row(b));
+                    mfma6_16x16x32(acc[2][nt], acc[3][nt], f, of_row(c), of_row(d));
                 }
-            }
-        }
+                __builtin_amdgcn_sched_barrier(0);  // rows and filter fragments are made as they are needed, not up front
+            };
+            products(0, r0, r1, r2, r3);
+            after_first();
+            const Row r4 = shifted(tx_c, std::integral_constant<int, 4>{});
+            products(1, r1, r2, r3, r4);
+            const Row r5 = shifted(tx_c, std::integral_constant<int, 5>{});
+            products(2, r2, r3, r4, r5);
+        };
+        phase(std::integral_constant<int, 1>{}, [] {});
+        phase(std::integral_constant<int, 0>{}, [] {});
+        phase(std::integral_constant<int, 2>{}, [&]() __attribute__((always_inline)) {
+#pragma unroll
+            for (int j = 0; j < ROWS; ++j) fetch(next, next_ok, j, 1, raw[j]);
+            fetch_halo(next, next_ok, raw_halo);
+        });
+
         done = here, have_done = true;
         done_special = w_special || __builtin_amdgcn_ballot_w64(!bf16_pairs_finite(magnitude)) != 0;
-        here = next;
+        here = next, item = next_index;
     }
     if (have_done) write_item(done, done_special);
 }
