@@ -463,7 +463,7 @@ def test_fconv_affine_relu_equals_separate_layers(dab, affine, relu, bias):
 @pytest.mark.parametrize("n,h,w,pad,cout,bias,affine,relu", [
     (24, 112, 112, 1, 32, False, True, True),   # the three-convolution stem's second convolution
     (22, 112, 112, 1, 64, True, False, False),  # its third
-    (99, 59, 46, 2, 32, True, True, False),     # 16 929 tiles of 16 pixels: the last work item is one tile, pad 2
+    (99, 59, 46, 2, 32, True, True, False),     # 61 output rows: the last column of four tiles is one row high; pad 2
     (25, 114, 114, 0, 64, False, False, True),  # no padding
 ])
 def test_fconv_3x3_over_32_channels_on_split_operands(dab, n, h, w, pad, cout, bias, affine, relu):
@@ -522,16 +522,21 @@ def test_fconv_3x3_over_32_channels_on_split_operands(dab, n, h, w, pad, cout, b
     goti = gpu(xi, wi).cpu().numpy()
     for i in (0, n - 1):
         np.testing.assert_array_equal(goti[i], cpu(xi[i], wi))
-    # a NaN pixel, an infinity in one channel, an infinity in a weight (its products with the image's zeros are NaN)
+    # a NaN pixel and an infinity in one channel (the work items they touch are made again the slow way, the others are
+    # not: one pixel beside a tile and one in a corner among them), then also an infinity in a weight (its products with
+    # the image's zeros are NaN; every work item the slow way)
     xi[0, h // 2, w // 3, :] = np.nan
     xi[-1, h // 3, w // 2, 5] = np.inf
     xi[1, 0, 0, 7] = -np.inf
-    wi[3, 1, 1, 9] = np.inf
-    with np.errstate(invalid="ignore"):
-        want = f64(xi, wi)
-    goti = gpu(xi, wi).cpu().numpy()
-    np.testing.assert_array_equal(np.isnan(goti), np.isnan(want))
-    np.testing.assert_array_equal(goti[~np.isnan(want)], want[~np.isnan(want)].astype(np.float32))
+    xi[2, 5, 16 - pad, 3] = np.inf  # the first pixel right of the first tile's sixteen: that tile sees it through its halo only
+    for weight_too in (False, True):
+        if weight_too:
+            wi[3, 1, 1, 9] = np.inf
+        with np.errstate(invalid="ignore"):
+            want = f64(xi, wi)
+        goti = gpu(xi, wi).cpu().numpy()
+        np.testing.assert_array_equal(np.isnan(goti), np.isnan(want))
+        np.testing.assert_array_equal(goti[~np.isnan(want)], want[~np.isnan(want)].astype(np.float32))
 
 
 def test_fconv_ramp_cases_of_reference_tests(dab):
