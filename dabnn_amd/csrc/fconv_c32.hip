@@ -163,6 +163,38 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                 as[nt][0] = fa.x, as[nt][1] = fa.y, as[nt][2] = fa.z, as[nt][3] = fa.w;
                 bb[nt][0] = fb.x, bb[nt][1] = fb.y, bb[nt][2] = fb.z, bb[nt][3] = fb.w;
             }
+            // bias, Affine and Relu each over all of the item's values under one test of its wave-uniform flag (tested
+            // per value they become a select per value and stage: 9 instead of 5 instructions per value)
+            {
+#pragma clang fp contract(off)
+                if (p.bias) {
+#pragma unroll
+                    for (int t = 0; t < PT; ++t)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[t][nt][e] = acc[t][nt][e] + bs[nt][e];
+                }
+                if (p.aff_a) {
+#pragma unroll
+                    for (int t = 0; t < PT; ++t)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float prod = as[nt][e] * acc[t][nt][e];
+                                acc[t][nt][e] = prod + bb[nt][e];
+                            }
+                }
+                if (p.relu) {
+#pragma unroll
+                    for (int t = 0; t < PT; ++t)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[t][nt][e] = acc[t][nt][e] < 0.f ? 0.f : acc[t][nt][e];  // std::max(v, 0.f): a NaN stays
+                }
+            }
             // a pixel's channel tiles one after the other: its 64-byte pieces complete 128-byte lines while they are
             // still in the write path
 #pragma unroll
@@ -170,12 +202,9 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                 if (at.oy0 + t >= p.oh) continue;
                 const size_t m = ((size_t)at.img * p.oh + at.oy0 + t) * p.ow + at.xt * 16 + f_i;
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = finish(acc[t][nt][e], bs[nt][e], as[nt][e], bb[nt][e]);
-                    *reinterpret_cast<float4 *>(p.out + m * COUT + 4 * g_now + nt * 16) = make_float4(v[0], v[1], v[2], v[3]);
-                }
+                for (int nt = 0; nt < NT; ++nt)
+                    *reinterpret_cast<float4 *>(p.out + m * COUT + 4 * g_now + nt * 16) =
+                        make_float4(acc[t][nt][0], acc[t][nt][1], acc[t][nt][2], acc[t][nt][3]);
             }
         } else {
             // The item is made again, one tile and one tap at a time, with the split that keeps an infinity or a NaN
