@@ -13,6 +13,8 @@ from .ops import (  # noqa: F401
     affine_inplace,
     ave_pool,
     ave_pool2_fconv1x1,
+    global_ave_pool_fconv1x1,
+    global_ave_pool_fconv1x1_takes,
     bconv_3x3,
     bconv_3x3_affine_add,
     bconv_3x3_affine_add_sign,

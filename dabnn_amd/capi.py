@@ -62,6 +62,8 @@ SIGNATURES = {
     "dab_fconv": (_i, [_vp, _i, _i, _i, _i, _vp, _vp] + [_i] * 9 + [_vp, _vp]),
     "dab_fconv_affine_relu": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp] + [_i] * 10 + [_vp, _vp]),
     "dab_ave_pool2_fconv1x1": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "dab_global_ave_pool_fconv1x1": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp]),
+    "dab_global_ave_pool_fconv1x1_takes": (_i, [_i] * 5),
     "dab_fconv_maxpool": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp] + [_i] * 10 + [_vp, _vp, _vp, _vp]),
     "dab_fconv_maxpool_carry_floats": (_i64, [_i] * 13),
     "dab_fconv_maxpool_pays": (_i, [_i] * 13),

@@ -374,6 +374,86 @@ __global__ __launch_bounds__(256) void fconv_gemv_kernel(const FconvArgs p) {
     }
 }
 
+// The same at the end of a net: a global AvePool (one window over the whole h x w image) and the classifier's 1x1
+// convolution in one launch, for the few images of a small batch.  Block (b, img) first averages image img into LDS --
+// thread t sums channels 4t .. 4t + 3 over the taps in ave_pool's order with ave_pool's rounding, so the pooled blob it
+// writes (block 0 of the image) is the one dab_ave_pool writes -- and then its four waves make kGlobalPoolChannels output
+// channels each, with fconv_gemv_kernel's arithmetic (lanes stride over the depth, sums added across the wave).  The
+// weights are asked for before the image: the two round trips to memory overlap.
+constexpr int kGlobalPoolChannels = 4;  // output channels per wave
+constexpr int kGlobalPoolTaps = 64;     // h * w at most
+constexpr int kGlobalPoolDepth4 = 256;  // c / 4 at most
+// D4: float4 of the depth per lane (c <= 256 * D4); U: taps asked for at once (49: a 7x7 window in one round trip)
+template <int D4, int U>
+__global__ __launch_bounds__(256) void global_avepool_gemv_kernel(const FconvArgs p) {
+    constexpr int CH = kGlobalPoolChannels;
+    __shared__ float4 pooled4[kGlobalPoolDepth4];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, img = blockIdx.y;
+    const int k4n = p.K >> 2, taps = p.h * p.wd;
+    const int co0 = (blockIdx.x * 4 + wave) * CH;
+    float4 wv[CH][D4];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+        const int co = co0 + j < p.cout ? co0 + j : p.cout - 1;  // a valid row; its sum is not stored
+        const float4 *w4 = reinterpret_cast<const float4 *>(p.w + (size_t)co * p.K);
+#pragma unroll
+        for (int i = 0; i < D4; ++i) wv[j][i] = lane + 64 * i < k4n ? w4[lane + 64 * i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if ((int)threadIdx.x < k4n) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(p.x) + (size_t)img * taps * k4n + threadIdx.x;
+        float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int t0 = 0; t0 < taps; t0 += U) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = x4[(size_t)(t0 + u < taps ? t0 + u : taps - 1) * k4n];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (t0 + u < taps) {
+#pragma clang fp contract(off)
+                    sum.x = sum.x + v[u].x, sum.y = sum.y + v[u].y, sum.z = sum.z + v[u].z, sum.w = sum.w + v[u].w;
+                }
+            }
+        }
+        const float d = (float)taps;
+        const float4 r = make_float4(__fdiv_rn(sum.x, d), __fdiv_rn(sum.y, d), __fdiv_rn(sum.z, d), __fdiv_rn(sum.w, d));
+        pooled4[threadIdx.x] = r;
+        if (blockIdx.x == 0) reinterpret_cast<float4 *>(p.pooled)[(size_t)img * k4n + threadIdx.x] = r;
+    }
+    __syncthreads();
+    float acc[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) acc[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < D4; ++i) {
+        if (lane + 64 * i < k4n) {
+            const float4 xv = pooled4[lane + 64 * i];
+#pragma unroll
+            for (int j = 0; j < CH; ++j) acc[j] += wv[j][i].x * xv.x + wv[j][i].y * xv.y + wv[j][i].z * xv.z + wv[j][i].w * xv.w;
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) acc[j] += __shfl_xor(acc[j], d, 64);
+    }
+    if (lane == 0) {
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            const int co = co0 + j;
+            if (co >= p.cout) break;
+            float v = acc[j];
+            if (p.bias) v = v + p.bias[co];
+            if (p.aff_a) {
+                const float prod = p.aff_a[co] * v;
+                v = prod + p.aff_b[co];
+            }
+            if (p.relu) v = v < 0.f ? 0.f : v;
+            p.out[(size_t)img * p.cout + co] = v;
+        }
+    }
+}
+
 // ---------------------------------------------------------------- elementwise
 // Affine.cpp:10-23.  Multiply and add are kept as two roundings, as the
 // reference's x86 build does, so results match it bit for bit.
@@ -646,6 +726,43 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
             DAB_FCONV_LAUNCH(128, 128, 16, 1, 1);
     }
 #undef DAB_FCONV_LAUNCH
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
+// Whether dab_global_ave_pool_fconv1x1 takes the shapes: the few images of a small batch (more of them are a matrix
+// product, which the pooling kernel and fconv_kernel do better), a window and a depth that fit the kernel's registers
+// and LDS, 16-byte rows.
+extern "C" int dab_global_ave_pool_fconv1x1_takes(int n, int h, int w, int c, int cout) {
+    using namespace dab;
+    return n >= 1 && n <= 8 && h >= 1 && w >= 1 && h * w <= kGlobalPoolTaps && c >= 4 && c % 4 == 0 &&
+           c / 4 <= kGlobalPoolDepth4 && cout >= 64;
+}
+
+extern "C" int dab_global_ave_pool_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                            const float *aff_a, const float *aff_b, int relu, int cout, float *pooled,
+                                            float *out, dab_stream_t stream) {
+    using namespace dab;
+    const char *fn = "dab_global_ave_pool_fconv1x1";
+    DAB_REQUIRE(x && wgt && pooled && out, "%s: null pointer", fn);
+    DAB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && cout > 0, "%s: non-positive dimension", fn);
+    DAB_REQUIRE((aff_a == nullptr) == (aff_b == nullptr), "%s: affine needs both coefficient vectors", fn);
+    if (!dab_global_ave_pool_fconv1x1_takes(n, h, w, c, cout) ||
+        (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt) | reinterpret_cast<uintptr_t>(pooled)) % 16 != 0)
+        return fail(DAB_EUNSUPPORTED, "%s: needs n <= 8, h * w <= %d, c %% 4 == 0, c <= %d, cout >= 64 and 16-byte aligned buffers", fn,
+                    kGlobalPoolTaps, 4 * kGlobalPoolDepth4);
+    FconvArgs a = {};
+    a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.relu = relu, a.out = out, a.pooled = pooled;
+    a.n = n, a.h = h, a.wd = w, a.c = c, a.cout = cout, a.K = c, a.M = n;
+    const unsigned blocks = (unsigned)((cout + 4 * kGlobalPoolChannels - 1) / (4 * kGlobalPoolChannels));
+    const dim3 grid(blocks, (unsigned)n);
+    hipStream_t s = as_stream(stream);
+    if (c <= 512 && h * w <= 49)
+        hipLaunchKernelGGL((global_avepool_gemv_kernel<2, 49>), grid, dim3(256), 0, s, a);
+    else if (c <= 512)
+        hipLaunchKernelGGL((global_avepool_gemv_kernel<2, 32>), grid, dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL((global_avepool_gemv_kernel<4, 32>), grid, dim3(256), 0, s, a);
     DAB_LAUNCH_CHECK();
     return DAB_OK;
 }

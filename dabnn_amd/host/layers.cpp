@@ -193,7 +193,7 @@ void FloatConv::check_operands() const {
 
 void FloatConv::forward_impl() const {
     if (fused_pool_input) {
-        dab_check(dab_ave_pool2_fconv1x1(
+        dab_check((fused_pool_global ? dab_global_ave_pool_fconv1x1 : dab_ave_pool2_fconv1x1)(
             static_cast<const float *>(fused_pool_input->dev), fused_pool_input->n, fused_pool_input->h, fused_pool_input->w,
             fused_pool_input->c, static_cast<const float *>(weight_mat->dev),
             bias_mat ? static_cast<const float *>(bias_mat->dev) : nullptr,
@@ -228,7 +228,8 @@ std::string FloatConv::to_str() const {
        << "x" << weight_mat->h << "x" << weight_mat->w;
     if (fused_a) ss << " + Affine";
     if (fused_relu) ss << " + Relu";
-    if (fused_pool_input) ss << ", AvePool 2x2 of " << fused_pool_input->h << "x" << fused_pool_input->w << " inside";
+    if (fused_pool_input)
+        ss << ", AvePool " << (fused_pool_global ? "over all" : "2x2") << " of " << fused_pool_input->h << "x" << fused_pool_input->w << " inside";
     if (fused_maxpool_out) ss << " + MaxPool 3x3 stride 2" << (fused_maxpool_sign ? " + Sign" : "");
     return ss.str();
 }

@@ -50,6 +50,8 @@ class BNN_API FloatConv : public Layer {
     // Set by Net::prepare for a 1x1 convolution that reads the output of an AvePool 2x2 stride 2: the pool's input.
     // The layer then pools it itself, writes the pooled blob (input_mat) as a side product and convolves it.
     MatP fused_pool_input;
+    // The same for a global AvePool (one window over the whole image) at small batch: fused_pool_input is its input.
+    bool fused_pool_global = false;
     // Set by Net::prepare when a MaxPool 3x3 stride 2 pad 1 is the only reader of the output: the pool's output blob,
     // the packed copy of it a direct BinConv wants (or null) and the workspace of the one-pass kernel.  output_mat is
     // null then: the convolution's result is never written.

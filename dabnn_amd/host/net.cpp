@@ -385,10 +385,13 @@ void Net::fuse_binconv_epilogues() {
 
     for (size_t i = 0; i + 1 < layers.size(); ++i) {
         auto pool = std::dynamic_pointer_cast<AvePool>(layers[i]);
-        if (!pool || pool->kernel_h != 2 || pool->kernel_w != 2 || pool->stride_h != 2 || pool->stride_w != 2 ||
-            pool->pad_h != 0 || pool->pad_w != 0 || pool->input_mat->c % 4 != 0 || pool->input_mat->h < 2 ||
-            pool->input_mat->w < 2)
-            continue;
+        if (!pool || pool->pad_h != 0 || pool->pad_w != 0 || pool->input_mat->c % 4 != 0) continue;
+        const bool two_by_two = pool->kernel_h == 2 && pool->kernel_w == 2 && pool->stride_h == 2 && pool->stride_w == 2 &&
+                                pool->input_mat->h >= 2 && pool->input_mat->w >= 2;
+        // one window over the whole image (the pool before a classifier); whether the one-launch form covers the shapes
+        // is asked below, when the convolution is known
+        const bool global = !two_by_two && pool->kernel_h == pool->input_mat->h && pool->kernel_w == pool->input_mat->w;
+        if (!two_by_two && !global) continue;
         // the one reader of the pooled blob must be a 1x1 FloatConv, with nothing in between that rewrites the pool's input
         size_t j = i + 1;
         bool ok = true;
@@ -406,7 +409,11 @@ void Net::fuse_binconv_epilogues() {
             if (contains(rd, pool->output_mat.get())) ok = false;  // someone else wants the pooled blob at its own time
         }
         if (!ok) continue;
+        if (global && !dab_global_ave_pool_fconv1x1_takes(pool->input_mat->n, pool->input_mat->h, pool->input_mat->w,
+                                                          pool->input_mat->c, fc->output_mat->c))
+            continue;
         fc->fused_pool_input = pool->input_mat;
+        fc->fused_pool_global = global;
         layers.erase(layers.begin() + i);
         --i;
     }

@@ -291,6 +291,33 @@ def ave_pool2_fconv1x1(x, weight, bias, a, b, relu):
     return pooled, out
 
 
+def global_ave_pool_fconv1x1(x, weight, bias, a, b, relu):
+    """Global AvePool (one h x w window) + 1x1 FpConv2D (+ Affine + Relu) in one launch; returns (pooled, out)."""
+    _need(x, torch.float32, "x")
+    _need(weight, torch.float32, "weight")
+    n, h, w, c = x.shape
+    cout = weight.shape[0]
+    if weight.numel() != cout * c:
+        raise capi.DabError(capi.DAB_EINVAL, "global_ave_pool_fconv1x1: weight must be [cout, 1, 1, c]")
+    def opt(t, name):
+        if t is None:
+            return None
+        _need(t, torch.float32, name)
+        if t.numel() != cout:
+            raise capi.DabError(capi.DAB_EINVAL, "global_ave_pool_fconv1x1: %s does not match the channel count" % name)
+        return _ptr(t)
+    pooled = _empty((n, 1, 1, c), torch.float32, x.device)
+    out = _empty((n, 1, 1, cout), torch.float32, x.device)
+    check(lib.dab_global_ave_pool_fconv1x1(_ptr(x), n, h, w, c, _ptr(weight), opt(bias, "bias"), opt(a, "a"), opt(b, "b"),
+                                           int(bool(relu)), cout, _ptr(pooled), _ptr(out), _stream()))
+    return pooled, out
+
+
+def global_ave_pool_fconv1x1_takes(n, h, w, c, cout):
+    """Whether global_ave_pool_fconv1x1 covers the shapes (small batch, window and depth within the kernel's limits)."""
+    return bool(lib.dab_global_ave_pool_fconv1x1_takes(n, h, w, c, cout))
+
+
 def fconv_maxpool(x, weight, bias, a, b, relu, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h=1, dil_w=1, want_sign=False):
     """FpConv2D (+ Affine + Relu) and MaxPool 3x3 stride 2 pad 1 in one pass; returns (pooled, pack_mat of it or None)."""
     _need(x, torch.float32, "x")

@@ -245,6 +245,21 @@ DAB_API int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, c
                                    dab_stream_t stream);
 
 /*
+ * A global AvePool -- one h x w window, stride 1, no padding, a 1 x 1 result per image (ave_pool_fallback,
+ * dabnn/layers/AvePool.cpp:84-123; Net::prepare builds the layer at dabnn/net.cpp:221-229) -- followed by a 1x1
+ * FpConv2D (dabnn/fconv.h:14-76) and the optional Affine and Relu of dab_fconv_affine_relu, in one launch: the end of
+ * a classifier at small batch.  pooled [n][1][1][c] receives the pooled tensor exactly as dab_ave_pool writes it, out
+ * [n][1][1][cout] the convolution of it exactly as dab_fconv_affine_relu computes it from that tensor.  wgt is
+ * [cout][1][1][c].  dab_global_ave_pool_fconv1x1_takes returns 1 for the shapes the launch covers (n <= 8,
+ * h * w <= 64, c a multiple of 4 up to 1024, cout >= 64); others, and x, wgt or pooled not 16-byte aligned, are
+ * DAB_EUNSUPPORTED: the two separate calls serve them.
+ */
+DAB_API int dab_global_ave_pool_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
+                                         const float *a, const float *b, int relu, int cout, float *pooled, float *out,
+                                         dab_stream_t stream);
+DAB_API int dab_global_ave_pool_fconv1x1_takes(int n, int h, int w, int c, int cout);
+
+/*
  * FpConv2D (dabnn/fconv.h:14-76) with the optional Affine and Relu of dab_fconv_affine_relu, followed by MaxPool 3x3,
  * stride 2, pad 1 (max_pool_fallback, dabnn/layers/MaxPool.cpp:209-246), in one pass that never writes the
  * convolution's output: the stem of a Bi-Real-style net.  pooled [n][oh/2][ow/2][cout] receives what dab_max_pool

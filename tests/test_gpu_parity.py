@@ -601,6 +601,47 @@ def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine)
         dab.ave_pool2_fconv1x1(dev_f(x[..., :3].copy()), dev_f(wgt[..., :3].copy()), None, None, None, False)
 
 
+@pytest.mark.parametrize("n,h,w,c,cout,bias,affine,relu", [
+    (1, 7, 7, 512, 1000, True, False, False),   # the end of Bi-Real-18 at batch 1
+    (8, 7, 7, 512, 1000, False, False, False),  # the most images it takes
+    (3, 8, 8, 1024, 64, True, True, True),      # the deepest and the largest window it takes, the fewest channels
+    (2, 1, 1, 4, 77, False, True, False),       # no pooling to speak of; a ragged last block
+    (5, 5, 3, 36, 100, True, False, True),      # a depth that leaves most lanes idle
+])
+def test_global_ave_pool_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, bias, affine, relu):
+    """A global AvePool and the classifier behind it in one launch (small batch): the pooled tensor is bit for bit what
+    ave_pool writes and what the CPU restatement computes, the result bit for bit what fconv_affine_relu makes of it
+    and within the float tolerance of the CPU layers."""
+    assert dab.global_ave_pool_fconv1x1_takes(n, h, w, c, cout)
+    r = rng(47)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    x[0, 0, 0, :4] = [0.0, -0.0, 1e-40, -1e-40]
+    wgt = (r.standard_normal((cout, 1, 1, c)) / np.sqrt(c)).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32)
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    args = (dev_f(bv) if bias else None, dev_f(a) if affine else None, dev_f(b) if affine else None, relu)
+    pooled, out = dab.global_ave_pool_fconv1x1(dev_f(x), dev_f(wgt), *args)
+    want_pooled = dab.ave_pool(dev_f(x), h, w, 0, 0, 1, 1)
+    want_out = dab.fconv_affine_relu(want_pooled, dev_f(wgt), *args, 1, 1, 0, 0, 1, 1)
+    assert pooled.shape == (n, 1, 1, c) and out.shape == (n, 1, 1, cout)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want_pooled.cpu().numpy())
+    np.testing.assert_array_equal(out.cpu().numpy(), want_out.cpu().numpy())
+    cpu_pooled = np.stack([orc.ave_pool(img, h, w, 0, 0, 1, 1) for img in x])
+    np.testing.assert_array_equal(pooled.cpu().numpy(), cpu_pooled)
+    for i in (0, n - 1):
+        y = orc.fconv(cpu_pooled[i], wgt, bv if bias else None, 1, 1, 0, 0, 1, 1)
+        if affine:
+            y = orc.affine_inplace(y.copy(), a, b)
+        if relu:
+            y = np.maximum(y, 0)
+        np.testing.assert_allclose(out.cpu().numpy()[i], y, rtol=RTOL, atol=RTOL * np.abs(y).max())
+    # shapes it leaves to the two separate calls
+    for shape in [(9, 7, 7, 512, 1000), (1, 9, 8, 512, 1000), (1, 7, 7, 510, 1000), (1, 7, 7, 2048, 1000), (1, 7, 7, 512, 10)]:
+        assert not dab.global_ave_pool_fconv1x1_takes(*shape)
+    with pytest.raises(RuntimeError):
+        dab.global_ave_pool_fconv1x1(dev_f(np.zeros((9, h, w, c), np.float32)), dev_f(wgt), None, None, None, False)
+
+
 @pytest.mark.parametrize("n,h,w,c,k,pad,stride,dil,cout,bias,affine,relu", [
     # output width 28, 56, 112 (bands of 16, 8, 4 rows), one band per image and several, three-channel images and
     # multiples of four channels, a depth that is no multiple of the slice, two channel tiles, a ragged channel tile

@@ -178,8 +178,9 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem, batch):
     # down-sampling blocks are fused too, behind their shortcut branch
     assert sum("+ Sign" in d for d in descs) == 15 and sum("packed input from its producer" in d for d in descs) == 16
     assert sum("+ Affine + Add" in d for d in descs) == 16 and not any(d.startswith("Add") for d in descs)
-    # the three shortcut branches pool inside their 1x1 convolution; only the global pool is left as a layer
-    assert sum("AvePool 2x2 of" in d for d in descs) == 3 and sum(d.startswith("AvePool") for d in descs) == 1
+    # the three shortcut branches pool inside their 1x1 convolution, and at this batch the classifier does too
+    assert sum("AvePool 2x2 of" in d for d in descs) == 3 and not any(d.startswith("AvePool") for d in descs)
+    assert sum("AvePool over all of 7x7 inside" in d for d in descs) == 1
     for i in range(batch):
         assert check_every_segment(n, layers, inits, i) >= 20
         assert check_packed_inputs(n, layers, i) == 16
@@ -199,6 +200,8 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem, batch):
     # kernel's at this size, with the MaxPool (and the sign bits of its result) behind it
     assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == (0 if stem else 1)
     assert sum(d.startswith("MaxPool") for d in descs) == (1 if stem else 0)
+    # and the global pool is a launch of its own before the classifier's matrix product
+    assert sum(d.startswith("AvePool") for d in descs) == 1 and not any("AvePool over all" in d for d in descs)
     big.close()
 
 
