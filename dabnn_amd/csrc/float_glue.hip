@@ -789,6 +789,13 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
     if (M >= (1ll << 31) - 128 || (long long)n * h * w * c >= (1ll << 31))
         return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
     a.M = (int)M;
+    if (M <= 8 && cout >= 64) {
+        // a handful of pooled pixels: dab_fconv_affine_relu makes them with its matrix-vector kernel, whose sums are
+        // added in another order than a tile's -- two launches, so that the result stays what the two calls give
+        int rc = dab_ave_pool(x, n, h, w, c, 2, 2, 0, 0, 2, 2, pooled, stream);
+        if (rc != DAB_OK) return rc;
+        return dab_fconv_affine_relu(pooled, n, a.oh, a.ow, c, wgt, bias, aff_a, aff_b, relu, 1, 1, 0, 0, 1, 1, 1, 1, cout, out, stream);
+    }
     a.div_ow = FastDiv((uint32_t)a.ow), a.div_oh = FastDiv((uint32_t)a.oh);
     a.kw = 1, a.dil_h = 1, a.dil_w = 1;
     a.div_c = FastDiv((uint32_t)c), a.div_kw = FastDiv(1u);

@@ -582,7 +582,10 @@ def test_affine_add_bit_exact(dab):
                                                  # slices), more than 128 output channels (64 rows x 256 columns), the
                                                  # latter with a ragged last tile both ways
                                                  (48, 56, 56, 64, 128, True), (170, 28, 28, 128, 256, False),
-                                                 (97, 30, 30, 64, 200, True), (256, 14, 14, 256, 512, True)])
+                                                 (97, 30, 30, 64, 200, True), (256, 14, 14, 256, 512, True),
+                                                 # eight pooled pixels or fewer and 64 output channels or more: the
+                                                 # convolution alone would be the matrix-vector kernel's
+                                                 (1, 4, 9, 20, 242, False), (2, 2, 5, 64, 64, True)])
 def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine):
     """The shortcut branch of a down-sampling block in one launch: the pooled tensor is bit for bit what ave_pool
     writes (and what the CPU restatement computes), the convolution bit for bit what fconv_affine_relu makes of it."""
