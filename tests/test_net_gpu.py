@@ -258,6 +258,34 @@ class CachedBlobs:
 
 
 @pytest.mark.parametrize("stem", [False, True])
+def test_bireal18_batches_between_the_benchmarks_match_cpu(mods, stem):
+    """Which kernel runs a layer changes with the batch (the depth-splitting kernel for small problems, the one-pass
+    stem from a handful of images on, the split-operand convolutions over 32 channels from batch 21, the second builds
+    of the unit kernel): batch sizes on both sides of those switches, every layer group of the first and the last image
+    against the CPU layers fed with the device's own blobs, and the same logits from a second run and from the graph."""
+    import torch
+    df, models, net = mods
+    layers, inits, inputs = models.bireal18(31, stem=stem)
+    buf = df.write_model(layers, inits, inputs)
+    for batch in (3, 5, 9, 17, 20, 21, 33, 100, 168):
+        n = net.Net(batch=batch).read_buf(buf)
+        gone = blobs_not_produced(n, layers)
+        x = torch.randn((batch, 224, 224, 3), generator=torch.Generator().manual_seed(batch)).cuda()
+        n.run(x)
+        cached = CachedBlobs(n)
+        for i in (0, batch - 1):
+            assert check_every_segment(cached, layers, inits, i, gone) >= 19, batch
+            assert check_packed_inputs(cached, layers, i) == 16, batch
+        first = cached.get_blob("logits").copy()
+        n.run(x)
+        n.run(x)
+        np.testing.assert_array_equal(n.get_blob("logits"), first, err_msg="batch %d" % batch)
+        n.close()
+        del x
+        torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("stem", [False, True])
 def test_bireal18_batch256_matches_cpu(mods, stem):
     """The benchmark's throughput configuration, both stems: at batch 256 other kernels run than at batch 2 or 64 (the
     four-waves-per-SIMD builds of the direct convolution with their epilogues, 64 x 256 tiles in the pooled shortcut
