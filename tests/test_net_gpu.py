@@ -257,6 +257,33 @@ class CachedBlobs:
         return getattr(self.n, attr)
 
 
+@pytest.mark.parametrize("seed", range(3))
+def test_miniature_nets_on_random_sizes(mods, seed):
+    """The two miniature graphs at seeded random image sizes and batches: every layer group of the first and the last
+    image against the CPU layers, packed inputs, and the same logits from a second run and from the graph."""
+    import torch
+    df, models, net = mods
+    r = np.random.default_rng(500 + seed)
+    for _ in range(6):
+        hw, batch = int(r.choice([8, 12, 16, 20, 24, 32])), int(r.integers(1, 70))
+        dense = bool(r.integers(0, 2))
+        make = models.dense_bnn if dense else models.small_bnn
+        layers, inits, inputs = make(int(r.integers(0, 1000)), hw=hw)
+        case = "%s hw %d batch %d" % ("dense" if dense else "small", hw, batch)
+        n = net.Net(batch=batch).read_buf(df.write_model(layers, inits, inputs))
+        gone = blobs_not_produced(n, layers)
+        x = torch.randn((batch, hw, hw, 3), generator=torch.Generator().manual_seed(batch)).cuda()
+        n.run(x)
+        for i in sorted({0, batch - 1}):
+            assert check_every_segment(n, layers, inits, i, gone) >= 7, case
+            assert check_packed_inputs(n, layers, i) == 3, case
+        first = n.get_blob("logits").copy()
+        n.run(x)
+        n.run(x)
+        np.testing.assert_array_equal(n.get_blob("logits"), first, err_msg=case)
+        n.close()
+
+
 @pytest.mark.parametrize("stem", [False, True])
 def test_bireal18_batches_between_the_benchmarks_match_cpu(mods, stem):
     """Which kernel runs a layer changes with the batch (the depth-splitting kernel for small problems, the one-pass
