@@ -42,6 +42,12 @@ bool fconv_c32_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int 
 int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias, const float *aff_a,
                   const float *aff_b, int relu, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
                   int dil_w, int cout, int oh, int ow, float *out, hipStream_t s);
+bool fconv_c32_pool_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
+                          int dil_w, int cout, int oh, int ow);
+long long fconv_c32_pool_workspace_floats(int n, int oh, int ow, int cout);
+int fconv_c32_pool_run(const float *x, int n, int h, int w, const float *wgt, const float *bias, const float *aff_a,
+                       const float *aff_b, int relu, int pad_h, int pad_w, int cout, int oh, int ow, float *pooled,
+                       uint64_t *pooled_packed, float *work, hipStream_t s);
 
 // Output extent of a convolution / pooling window (common/Shaper.cpp:34-54).
 inline int out_dim(int in, int pad, int k, int dil, int stride) { return (in + 2 * pad - (dil * (k - 1) + 1)) / stride + 1; }

@@ -25,6 +25,8 @@ namespace dab {
 struct FconvC32Args {
     const float *x, *w, *bias, *aff_a, *aff_b;
     float *out;
+    float *brow, *bcol;  // POOL: every fourth output row and every sixteenth output column, for the pass that completes the pooling
+    uint64_t *bits;      // the completing pass: pack_mat of the pooled tensor, or null
     int relu;
     int h, wd, oh, ow, cout, pad_h, pad_w;
     uint32_t x_bytes;
@@ -37,7 +39,14 @@ struct FconvC32Args {
 constexpr int kC32Threads = 512, kC32PixelTiles = 4;
 constexpr uint32_t kC32Oob = 0x80000000u;  // beyond the descriptor (images here are shorter than 2^31 bytes)
 
-template <int NT, int KH, int KW>  // NT: 16-channel tiles of the output (cout = 16 * NT)
+// POOL: a MaxPool 3x3, stride 2, pad 1 (max_pool_fallback, dabnn/layers/MaxPool.cpp:209-246) follows and the convolution's
+// own result is not wanted.  A wave's column of four output rows x 16 pixels holds two pooled rows x eight pooled pixels:
+// it pools what it has -- rows as elementwise maxima of its accumulators, columns as maxima with the two neighbouring
+// lanes -- and writes that to p.out, now [n][oh / 2][ow / 2][cout].  What it lacks is the output row above the column
+// (for its first pooled row) and the output pixel left of it (for its first pooled pixel): every column also writes its
+// last output row to p.brow [n][oh / 4][ow][cout] and its last pixel of each row to p.bcol [n][oh / 4][ow / 16][4][cout],
+// and c32_pool_complete_kernel takes the maxima with those afterwards.  oh must be a multiple of 4.
+template <int NT, int KH, int KW, bool POOL = false>  // NT: 16-channel tiles of the output (cout = 16 * NT)
 __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Args p) {
     constexpr int TAPS = KH * KW, PT = kC32PixelTiles, COUT = 16 * NT;
     constexpr int ROW = TAPS * 32 + 8;     // bf16 elements per output channel in a plane
@@ -147,6 +156,28 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     fetch_halo(here, first + wave < last, raw_halo);
 
     f32x4w acc[PT][NT];
+    // max_pool's step: a later tap replaces the maximum only when it is greater (a NaN never is)
+    auto later_max = [](float m, float v) { return v > m ? v : m; };
+    // POOL: a tile column's two pooled rows for channel tile nt from the maxima over its output rows {0, 1} (v0) and
+    // {1, 2, 3} (v1): lane f (even) takes the maximum over pixels f - 1, f, f + 1 of the tile and stores pooled pixel f / 2
+    auto pool_store = [&](const Place &at, int nt, int g_now, const f32x4w &v0, const f32x4w &v1) __attribute__((always_inline)) {
+        const int lowest = __float_as_int(-FLT_MAX);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const f32x4w &v = half ? v1 : v0;
+            float h[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float left = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x111, 0xf, 0xf, false));
+                const float right = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x101, 0xf, 0xf, false));
+                h[e] = later_max(later_max(later_max(-FLT_MAX, left), v[e]), right);
+            }
+            if (!(f_i & 1)) {
+                const size_t cell = ((size_t)at.img * (p.oh >> 1) + (at.oy0 >> 1) + half) * (p.ow >> 1) + at.xt * 8 + (f_i >> 1);
+                *reinterpret_cast<float4 *>(p.out + cell * COUT + nt * 16 + 4 * g_now) = make_float4(h[0], h[1], h[2], h[3]);
+            }
+        }
+    };
     // Writes the item at `at`, whose sums are in acc (special: an infinity or a NaN among its pixels or in the filters).
     auto write_item = [&](const Place &at, bool special) __attribute__((always_inline)) {
         int g_now = g;
@@ -195,6 +226,33 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                             for (int e = 0; e < 4; ++e) acc[t][nt][e] = acc[t][nt][e] < 0.f ? 0.f : acc[t][nt][e];  // std::max(v, 0.f): a NaN stays
                 }
             }
+            if constexpr (POOL) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    f32x4w v0, v1;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v0[e] = later_max(later_max(-FLT_MAX, acc[0][nt][e]), acc[1][nt][e]);
+                        v1[e] = later_max(later_max(later_max(-FLT_MAX, acc[1][nt][e]), acc[2][nt][e]), acc[3][nt][e]);
+                    }
+                    pool_store(at, nt, g_now, v0, v1);
+                    // the last row as it is; the last pixel of the four rows gathered into lanes 12..15 of each group
+                    float *row = p.brow + ((((size_t)at.img * p.row_groups + (at.oy0 >> 2)) * p.ow + at.xt * 16 + f_i) * COUT + nt * 16 + 4 * g_now);
+                    *reinterpret_cast<float4 *>(row) = make_float4(acc[3][nt][0], acc[3][nt][1], acc[3][nt][2], acc[3][nt][3]);
+                    float w[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int r2 = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[2][nt][e]), 0x101, 0xf, 0xf, true);  // lane 14 <- 15
+                        const int r1 = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[1][nt][e]), 0x102, 0xf, 0xf, true);  // lane 13 <- 15
+                        const int r0 = __builtin_amdgcn_update_dpp(0, __float_as_int(acc[0][nt][e]), 0x103, 0xf, 0xf, true);  // lane 12 <- 15
+                        w[e] = f_i == 15 ? acc[3][nt][e] : __int_as_float(f_i == 14 ? r2 : f_i == 13 ? r1 : r0);
+                    }
+                    if (f_i >= 12) {
+                        float *col = p.bcol + (((((size_t)at.img * p.row_groups + (at.oy0 >> 2)) * p.tiles_per_row + at.xt) * 4 + (f_i - 12)) * COUT + nt * 16 + 4 * g_now);
+                        *reinterpret_cast<float4 *>(col) = make_float4(w[0], w[1], w[2], w[3]);
+                    }
+                }
+            } else {
             // a pixel's channel tiles one after the other: its 64-byte pieces complete 128-byte lines while they are
             // still in the write path
 #pragma unroll
@@ -206,16 +264,21 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                     *reinterpret_cast<float4 *>(p.out + m * COUT + 4 * g_now + nt * 16) =
                         make_float4(acc[t][nt][0], acc[t][nt][1], acc[t][nt][2], acc[t][nt][3]);
             }
+            }
         } else {
             // The item is made again, one tile and one tap at a time, with the split that keeps an infinity or a NaN
             // whole in hi and takes copies with the non-finite values zeroed for the cross terms (Inf * 0 would make a
             // NaN of a sum that is an infinity).
 #pragma unroll 1
-            for (int t = 0; t < PT; ++t) {
-                if (at.oy0 + t >= p.oh) break;
-                const size_t m = ((size_t)at.img * p.oh + at.oy0 + t) * p.ow + at.xt * 16 + f_i;
+            for (int nt = 0; nt < NT; ++nt) {
+                const int co = nt * 16 + 4 * g_now;
+                const float4 bias = *reinterpret_cast<const float4 *>(per_channel[0] + co);
+                const float4 fa = *reinterpret_cast<const float4 *>(per_channel[1] + co);
+                const float4 fb = *reinterpret_cast<const float4 *>(per_channel[2] + co);
+                f32x4w v0 = f32x4w{-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX}, v1 = v0;
 #pragma unroll 1
-                for (int nt = 0; nt < NT; ++nt) {
+                for (int t = 0; t < PT; ++t) {
+                    if (at.oy0 + t >= p.oh) break;
                     f32x4w one = f32x4w{0.f, 0.f, 0.f, 0.f}, none = one;
 #pragma unroll 1
                     for (int tap = 0; tap < TAPS; ++tap) {
@@ -232,14 +295,24 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                         for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
                         mfma6_16x16x32(one, none, f, px, px);
                     }
-                    const int co = nt * 16 + 4 * g_now;
-                    const float4 bias = *reinterpret_cast<const float4 *>(per_channel[0] + co);
-                    const float4 fa = *reinterpret_cast<const float4 *>(per_channel[1] + co);
-                    const float4 fb = *reinterpret_cast<const float4 *>(per_channel[2] + co);
-                    *reinterpret_cast<float4 *>(p.out + m * COUT + co) =
-                        make_float4(finish(one[0], bias.x, fa.x, fb.x), finish(one[1], bias.y, fa.y, fb.y),
-                                    finish(one[2], bias.z, fa.z, fb.z), finish(one[3], bias.w, fa.w, fb.w));
+                    const float4 fin = make_float4(finish(one[0], bias.x, fa.x, fb.x), finish(one[1], bias.y, fa.y, fb.y),
+                                                   finish(one[2], bias.z, fa.z, fb.z), finish(one[3], bias.w, fa.w, fb.w));
+                    if constexpr (POOL) {
+                        const float fv[4] = {fin.x, fin.y, fin.z, fin.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (t <= 1) v0[e] = later_max(v0[e], fv[e]);
+                            if (t >= 1) v1[e] = later_max(v1[e], fv[e]);
+                        }
+                        const size_t group = (size_t)at.img * p.row_groups + (at.oy0 >> 2);
+                        if (t == PT - 1) *reinterpret_cast<float4 *>(p.brow + ((group * p.ow + at.xt * 16 + f_i) * COUT + co)) = fin;
+                        if (f_i == 15) *reinterpret_cast<float4 *>(p.bcol + (((group * p.tiles_per_row + at.xt) * 4 + t) * COUT + co)) = fin;
+                    } else {
+                        const size_t m = ((size_t)at.img * p.oh + at.oy0 + t) * p.ow + at.xt * 16 + f_i;
+                        *reinterpret_cast<float4 *>(p.out + m * COUT + co) = fin;
+                    }
                 }
+                if constexpr (POOL) pool_store(at, nt, g_now, v0, v1);
             }
         }
     };
@@ -356,6 +429,66 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     if (have_done) write_item(done, done_special);
 }
 
+// The pass behind fconv_c32_kernel<..., POOL>: a pooled cell of an even pooled row (the first of its tile column) takes
+// the maxima with the three output pixels above it, which are in the last row of the tile column above (brow); a cell
+// that is the first of its tile takes them with the output pixels left of it, the last pixels of the tile to the left
+// (bcol).  The other cells are final as they are.  SIGN: pack_mat of the pooled tensor (cout a multiple of 64) -- the 16
+// threads that hold the 64 channels of a word are one row of lanes, as in pool_vec4_kernel.
+struct C32PoolCompleteArgs {
+    float4 *pooled;
+    const float4 *brow, *bcol;
+    uint64_t *bits;
+    int ph, pw, c4, ow, groups, tiles;
+    uint32_t total;
+    FastDiv div_c4, div_pw, div_ph;
+};
+
+template <bool SIGN>
+__global__ __launch_bounds__(256) void c32_pool_complete_kernel(const C32PoolCompleteArgs p) {
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= p.total) return;
+    const uint32_t t = p.div_c4.div(idx);
+    const int ch = (int)(idx - t * (uint32_t)p.c4);
+    const uint32_t t2 = p.div_pw.div(t);
+    const int c = (int)(t - t2 * (uint32_t)p.pw);
+    const uint32_t img = p.div_ph.div(t2);
+    const int r = (int)(t2 - img * (uint32_t)p.ph), m = r >> 1;
+    auto later_max = [](float4 a, float4 v) {
+        return make_float4(v.x > a.x ? v.x : a.x, v.y > a.y ? v.y : a.y, v.z > a.z ? v.z : a.z, v.w > a.w ? v.w : a.w);
+    };
+    float4 v = p.pooled[idx];
+    bool changed = false;
+    if (!(r & 1) && m > 0) {
+        const float4 *row = p.brow + ((size_t)img * p.groups + (m - 1)) * p.ow * p.c4 + ch;
+#pragma unroll
+        for (int dx = -1; dx <= 1; ++dx) {
+            const int x = 2 * c + dx;
+            if ((unsigned)x < (unsigned)p.ow) v = later_max(v, row[(size_t)x * p.c4]);
+        }
+        changed = true;
+    }
+    if (!(c & 7) && c > 0) {
+        const float4 *col = p.bcol + ((((size_t)img * p.groups + m) * p.tiles + ((c >> 3) - 1)) * 4) * p.c4 + ch;
+        if (r & 1) {
+            v = later_max(later_max(later_max(v, col[p.c4]), col[2 * p.c4]), col[3 * p.c4]);
+        } else {
+            v = later_max(later_max(v, col[0]), col[p.c4]);
+        }
+        changed = true;
+    }
+    if (changed) p.pooled[idx] = v;
+    if constexpr (SIGN) {
+        const int part = (int)(idx & 15u);
+        const uint32_t nib = sign_nibble(v);
+        uint32_t lo = part < 8 ? nib << (4 * part) : 0u, hi = part >= 8 ? nib << (4 * (part - 8)) : 0u;
+        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+        if (part == 0) p.bits[idx >> 4] = ((uint64_t)hi << 32) | lo;
+    }
+}
+
 // Whether the shapes are this kernel's and the problem is large enough to fill its persistent waves (buffer alignment
 // aside, which only the call itself can check).
 bool fconv_c32_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
@@ -382,6 +515,7 @@ int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, 
     const int blocks = simd_count() / 4;  // one block of eight waves per CU (the filter planes take most of its LDS)
     FconvC32Args a;
     a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.out = out, a.relu = relu;
+    a.brow = nullptr, a.bcol = nullptr, a.bits = nullptr;
     a.h = h, a.wd = w, a.oh = oh, a.ow = ow, a.cout = cout, a.pad_h = pad_h, a.pad_w = pad_w;
     a.x_bytes = (uint32_t)((long long)n * h * w * 128);
     a.row_groups = (oh + kC32PixelTiles - 1) / kC32PixelTiles, a.tiles_per_row = ow / 16;
@@ -392,6 +526,55 @@ int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, 
     else
         hipLaunchKernelGGL((fconv_c32_kernel<4, 3, 3>), dim3(blocks), dim3(kC32Threads), 0, s, a);
     return hipGetLastError() == hipSuccess ? 1 : fail(DAB_EHIP, "fconv_c32: launch failed");
+}
+
+// The convolution with the MaxPool 3x3, stride 2, pad 1 behind it (fconv_c32_kernel<..., POOL> and the completing pass):
+// the shapes of fconv_c32_takes with an output height that is a multiple of 4.  workspace_floats: what `work` must hold.
+bool fconv_c32_pool_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
+                          int dil_w, int cout, int oh, int ow) {
+    return oh % 4 == 0 && fconv_c32_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, oh, ow) &&
+           (long long)n * (oh / 2) * (ow / 2) * (cout / 4) < (1ll << 32);
+}
+
+long long fconv_c32_pool_workspace_floats(int n, int oh, int ow, int cout) {
+    return (long long)n * (oh / 4) * ow * cout + (long long)n * (oh / 4) * (ow / 16) * 4 * cout;
+}
+
+// Returns 1 when it ran, 0 when the buffers are not 16-byte aligned (the caller takes another path), negative on failure.
+int fconv_c32_pool_run(const float *x, int n, int h, int w, const float *wgt, const float *bias, const float *aff_a,
+                       const float *aff_b, int relu, int pad_h, int pad_w, int cout, int oh, int ow, float *pooled,
+                       uint64_t *pooled_packed, float *work, hipStream_t s) {
+    uintptr_t align = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt) | reinterpret_cast<uintptr_t>(pooled) |
+                      reinterpret_cast<uintptr_t>(work);
+    if (bias) align |= reinterpret_cast<uintptr_t>(bias);
+    if (aff_a) align |= reinterpret_cast<uintptr_t>(aff_a) | reinterpret_cast<uintptr_t>(aff_b);
+    if (align % 16 != 0) return 0;
+    const int blocks = simd_count() / 4;
+    FconvC32Args a;
+    a.x = x, a.w = wgt, a.bias = bias, a.aff_a = aff_a, a.aff_b = aff_b, a.out = pooled, a.relu = relu;
+    a.brow = work, a.bcol = work + (size_t)n * (oh / 4) * ow * cout, a.bits = nullptr;
+    a.h = h, a.wd = w, a.oh = oh, a.ow = ow, a.cout = cout, a.pad_h = pad_h, a.pad_w = pad_w;
+    a.x_bytes = (uint32_t)((long long)n * h * w * 128);
+    a.row_groups = oh / kC32PixelTiles, a.tiles_per_row = ow / 16;
+    a.items = n * a.row_groups * a.tiles_per_row;
+    a.div_tiles_per_row = FastDiv((uint32_t)a.tiles_per_row), a.div_row_groups = FastDiv((uint32_t)a.row_groups);
+    if (cout == 32)
+        hipLaunchKernelGGL((fconv_c32_kernel<2, 3, 3, true>), dim3(blocks), dim3(kC32Threads), 0, s, a);
+    else
+        hipLaunchKernelGGL((fconv_c32_kernel<4, 3, 3, true>), dim3(blocks), dim3(kC32Threads), 0, s, a);
+    if (hipGetLastError() != hipSuccess) return fail(DAB_EHIP, "fconv_c32 (pooled): launch failed");
+    C32PoolCompleteArgs f;
+    f.pooled = reinterpret_cast<float4 *>(pooled), f.brow = reinterpret_cast<const float4 *>(a.brow);
+    f.bcol = reinterpret_cast<const float4 *>(a.bcol), f.bits = pooled_packed;
+    f.ph = oh / 2, f.pw = ow / 2, f.c4 = cout / 4, f.ow = ow, f.groups = a.row_groups, f.tiles = a.tiles_per_row;
+    f.total = (uint32_t)((long long)n * f.ph * f.pw * f.c4);
+    f.div_c4 = FastDiv((uint32_t)f.c4), f.div_pw = FastDiv((uint32_t)f.pw), f.div_ph = FastDiv((uint32_t)f.ph);
+    const unsigned grid = (f.total + 255u) / 256u;
+    if (pooled_packed)
+        hipLaunchKernelGGL(c32_pool_complete_kernel<true>, dim3(grid), dim3(256), 0, s, f);
+    else
+        hipLaunchKernelGGL(c32_pool_complete_kernel<false>, dim3(grid), dim3(256), 0, s, f);
+    return hipGetLastError() == hipSuccess ? 1 : fail(DAB_EHIP, "fconv_c32 (pooled): launch failed");
 }
 
 }  // namespace dab

@@ -664,6 +664,9 @@ extern "C" int64_t dab_fconv_maxpool_carry_floats(int n, int h, int w, int c, in
                                                   int stride_h, int stride_w, int dil_h, int dil_w, int cout) {
     dab::BandPlan b;
     if (n <= 0 || !dab::plan_bands(h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b)) return 0;
+    // the split-operand kernel's pooled form keeps a quarter of the output rows and a sixteenth of its columns instead
+    if (dab::fconv_c32_pool_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b.oh, b.ow))
+        return dab::fconv_c32_pool_workspace_floats(n, b.oh, b.ow, cout);
     return (int64_t)n * b.bands * b.pw * cout;
 }
 
@@ -678,8 +681,10 @@ extern "C" int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw
     // kernel gains a few per cent over full rounds and loses as much as the last round is empty (32 -> 64 channels at
     // 112 x 112, one pass against two launches: 127 / 128 us at 672 bands, 166 / 143 at 784, 166 / 166 at 896,
     // 205 / 187 at 1036): it runs when the last round leaves less than an eighth of all slots idle.
-    // 3x3 convolutions over 32 channels that are large enough for the split-operand kernel: that kernel and a separate
-    // MaxPool beat the one pass over im2col slices (32 -> 64 at 112 x 112, batch 256: 0.76 + 0.21 against 1.35 ms)
+    // 3x3 convolutions over 32 channels that are large enough for the split-operand kernel: its pooled form where the
+    // output height allows it; otherwise that kernel and a separate MaxPool beat the one pass over im2col slices
+    // (32 -> 64 at 112 x 112, batch 256: 0.76 + 0.21 against 1.35 ms)
+    if (dab::fconv_c32_pool_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b.oh, b.ow)) return 1;
     if (dab::fconv_c32_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b.oh, b.ow)) return 0;
     const long long blocks = (long long)n * b.bands * ((cout + dab::kBandChannels - 1) / dab::kBandChannels);
     const long long cus = dab::simd_count() / 4;
@@ -709,6 +714,12 @@ extern "C" int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, con
     if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wgt) | reinterpret_cast<uintptr_t>(pooled) |
          reinterpret_cast<uintptr_t>(carry)) % 16 != 0)
         return fail(DAB_EUNSUPPORTED, "%s: needs 16-byte aligned buffers", fn);
+    if (fconv_c32_pool_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, b.oh, b.ow)) {
+        // alignment of the optional vectors decides at the call: unaligned ones take the band kernel below
+        const int rc = fconv_c32_pool_run(x, n, h, w, wgt, bias, aff_a, aff_b, relu, pad_h, pad_w, cout, b.oh, b.ow, pooled,
+                                          pooled_packed, carry, as_stream(stream));
+        if (rc != 0) return rc < 0 ? rc : DAB_OK;
+    }
     const long long pooled_elems = (long long)n * b.ph * b.pw * cout;
     if ((long long)n * b.oh >= (1ll << 31) || pooled_elems >= (1ll << 33))
         return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);

@@ -474,10 +474,10 @@ def test_fconv_3x3_over_32_channels_on_split_operands(dab, n, h, w, pad, cout, b
     matrix cores with operands split in three (fp32 accuracy): within the float tolerance of the CPU layers on a sample
     of images and of a float64 convolution on all of them, exact on small integers, and an infinity or a NaN in the
     image comes out where IEEE arithmetic puts it (zero times infinity included: a zero weight)."""
-    # the size gate of the kernel, seen through the one entry point that reports it: these shapes no longer take the
-    # one-pass convolution + MaxPool
+    # with a MaxPool behind them these shapes take one pass at either size: the band kernel at batch 18, this kernel's
+    # pooled form where it is large enough
     if cout == 64 and pad == 1 and h == 112:
-        assert not dab.fconv_maxpool_pays(n, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
+        assert dab.fconv_maxpool_pays(n, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
         assert dab.fconv_maxpool_pays(18, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
     r = rng(61)
     x = r.standard_normal((n, h, w, 32)).astype(np.float32)
@@ -718,6 +718,73 @@ def test_fconv_maxpool_one_pass(dab, n, h, w, c, k, pad, stride, dil, cout, bias
     np.testing.assert_array_equal(pooled.cpu().numpy(), want)
     if sign:
         np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+
+
+@pytest.mark.parametrize("n,h,w,pad,cout,bias,affine,relu", [
+    (22, 112, 112, 1, 64, False, True, True),   # the three-convolution stem's last convolution and its MaxPool
+    (24, 112, 112, 1, 32, True, False, False),  # 32 output channels: no sign bits
+    (600, 28, 16, 1, 64, True, True, False),    # one tile per row: no tile to the left anywhere
+    (300, 28, 32, 1, 64, False, False, True),   # two tiles per row
+    (70, 110, 110, 2, 64, False, True, True),   # pad 2: a 112 x 112 output of a 110 x 110 image
+])
+def test_fconv_maxpool_over_32_channels_pools_in_registers(dab, n, h, w, pad, cout, bias, affine, relu):
+    """3x3 stride-1 convolutions over 32 channels that are large enough take the split-operand kernel also with a
+    MaxPool 3x3 stride 2 pad 1 behind them: a tile column pools what it holds and a second pass completes the cells
+    that need the row above or the pixel to the left.  Equal to max_pool_sign of the separate convolution on the
+    device (the same products, the same maxima), within the float tolerance of the CPU layers, exact on small
+    integers, and infinities and NaNs come out as the CPU layers put them."""
+    assert dab.fconv_maxpool_pays(n, h, w, 32, 3, 3, pad, pad, 1, 1, 1, 1, cout)
+    r = rng(63)
+    x = r.standard_normal((n, h, w, 32)).astype(np.float32)
+    wgt = (r.standard_normal((cout, 3, 3, 32)) / 17).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32) if bias else None
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    sign = cout % 64 == 0
+
+    def both(x, wgt, bv, a, b):
+        args = (dev_f(bv) if bias else None, dev_f(a) if affine else None, dev_f(b) if affine else None, relu)
+        pooled, packed = dab.fconv_maxpool(dev_f(x), dev_f(wgt), *args, 3, 3, pad, pad, 1, 1, 1, 1, want_sign=sign)
+        conv = dab.fconv_affine_relu(dev_f(x), dev_f(wgt), *args, 3, 3, pad, pad, 1, 1)
+        if sign:
+            want, want_packed = dab.max_pool_sign(conv, 3, 3, 1, 1, 2, 2)
+            assert torch.equal(packed, want_packed)
+            assert torch.equal(packed, dab.pack_mat(pooled))
+        else:
+            want = dab.max_pool(conv, 3, 3, 1, 1, 2, 2)
+        return pooled.cpu().numpy(), want.cpu().numpy()
+
+    def cpu(img, wgt, bv, a, b):
+        y = orc.fconv(img, wgt, bv, 3, 3, pad, pad, 1, 1)
+        if affine:
+            y = orc.affine_inplace(y.copy(), a, b)
+        if relu:
+            y = np.maximum(y, 0)
+        return orc.max_pool(y, 3, 3, 1, 1, 2, 2)
+
+    got, want = both(x, wgt, bv, a, b)
+    assert got.shape == (n, (h + 2 * pad - 2) // 2, (w + 2 * pad - 2) // 2, cout)
+    np.testing.assert_array_equal(got, want)
+    for i in (0, n - 1):
+        ref = cpu(x[i], wgt, bv, a, b)
+        np.testing.assert_allclose(got[i], ref, rtol=RTOL, atol=RTOL * np.abs(ref).max())
+    # small integers: exact; then an infinity, a NaN pixel and a NaN at a tile's edge
+    xi = r.integers(-3, 4, x.shape).astype(np.float32)
+    wi = r.integers(-2, 3, wgt.shape).astype(np.float32)
+    bi = r.integers(-5, 6, cout).astype(np.float32) if bias else None
+    ai, ci = r.integers(-2, 3, cout).astype(np.float32), r.integers(-9, 10, cout).astype(np.float32)
+    got, want = both(xi, wi, bi, ai, ci)
+    np.testing.assert_array_equal(got, want)
+    for i in (0, n - 1):
+        np.testing.assert_array_equal(got[i], cpu(xi[i], wi, bi, ai, ci))
+    xi[0, h // 2, w // 3, :] = np.nan
+    xi[-1, h // 3, w // 2, 5] = np.inf
+    xi[1, min(3, h - 1), min(15, w - 1), 7] = -np.inf
+    xi[2, min(4, h - 1), min(16 - pad, w - 1), 3] = np.nan
+    got, want = both(xi, wi, bi, ai, ci)
+    np.testing.assert_array_equal(got, want)
+    with np.errstate(invalid="ignore"):
+        for i in (0, 1, 2, n - 1):
+            np.testing.assert_array_equal(got[i], cpu(xi[i], wi, bi, ai, ci))
 
 
 def test_fconv_maxpool_rejects_other_shapes(dab):

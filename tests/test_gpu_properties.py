@@ -176,9 +176,9 @@ def test_fconv_maxpool_full_size_against_torch(dab, n, hw, c, cout, k, pad, stri
     a, b = torch.randn(cout, generator=gen).cuda(), torch.randn(cout, generator=gen).cuda()
     torch.backends.cudnn.allow_tf32 = False
     torch.backends.cuda.matmul.allow_tf32 = False
-    # the Net takes this pass for the 7x7 stem; the 3x3 convolution over 32 channels at this size goes to the
-    # split-operand kernel with a separate MaxPool instead, and the one-pass kernel stays callable
-    assert dab.fconv_maxpool_pays(n, hw, hw, c, k, k, pad, pad, stride, stride, 1, 1, cout) == (c == 3)
+    # the Net takes this pass for both stems: the band kernel for the 7x7 stem, the pooled form of the split-operand
+    # kernel for the 3x3 convolution over 32 channels at this size
+    assert dab.fconv_maxpool_pays(n, hw, hw, c, k, k, pad, pad, stride, stride, 1, 1, cout)
     ref = F.conv2d(x.permute(0, 3, 1, 2), w.permute(0, 3, 1, 2), None, stride=stride, padding=pad)
     ref = ref * a.view(1, -1, 1, 1) + b.view(1, -1, 1, 1)
     scale = ref.abs().max().item()
