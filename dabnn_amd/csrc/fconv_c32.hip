@@ -156,8 +156,21 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     fetch_halo(here, first + wave < last, raw_halo);
 
     f32x4w acc[PT][NT];
-    // max_pool's step: a later tap replaces the maximum only when it is greater (a NaN never is)
-    auto later_max = [](float m, float v) { return v > m ? v : m; };
+    // max_pool's step, `v > m ? v : m` from -FLT_MAX on, as the hardware's maximum: a NaN is passed over either way (the
+    // running maximum never is one); where +0 and -0 tie the hardware gives +0 and max_pool the earlier tap, which no
+    // comparison and no sign bit of the result can tell apart
+    // (the instructions by name: fmaxf would come with an instruction per operand that quiets signalling NaNs, which
+    // these values -- results of arithmetic -- never are)
+    auto later_max = [](float m, float v) {
+        float r;
+        asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(m), "v"(v));
+        return r;
+    };
+    auto max_of_three = [](float a, float b, float c) {
+        float r;
+        asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+        return r;
+    };
     // POOL: a tile column's two pooled rows for channel tile nt from the maxima over its output rows {0, 1} (v0) and
     // {1, 2, 3} (v1): lane f (even) takes the maximum over pixels f - 1, f, f + 1 of the tile and stores pooled pixel f / 2
     auto pool_store = [&](const Place &at, int nt, int g_now, const f32x4w &v0, const f32x4w &v1) __attribute__((always_inline)) {
@@ -170,7 +183,7 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
             for (int e = 0; e < 4; ++e) {
                 const float left = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x111, 0xf, 0xf, false));
                 const float right = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x101, 0xf, 0xf, false));
-                h[e] = later_max(later_max(later_max(-FLT_MAX, left), v[e]), right);
+                h[e] = max_of_three(left, v[e], right);
             }
             if (!(f_i & 1)) {
                 const size_t cell = ((size_t)at.img * (p.oh >> 1) + (at.oy0 >> 1) + half) * (p.ow >> 1) + at.xt * 8 + (f_i >> 1);
@@ -232,8 +245,8 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
                     f32x4w v0, v1;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        v0[e] = later_max(later_max(-FLT_MAX, acc[0][nt][e]), acc[1][nt][e]);
-                        v1[e] = later_max(later_max(later_max(-FLT_MAX, acc[1][nt][e]), acc[2][nt][e]), acc[3][nt][e]);
+                        v0[e] = later_max(acc[0][nt][e], acc[1][nt][e]);
+                        v1[e] = max_of_three(acc[1][nt][e], acc[2][nt][e], acc[3][nt][e]);
                     }
                     pool_store(at, nt, g_now, v0, v1);
                     // the last row as it is; the last pixel of the four rows gathered into lanes 12..15 of each group
