@@ -264,8 +264,9 @@ DAB_API int dab_global_ave_pool_fconv1x1_takes(int n, int h, int w, int c, int c
  * stride 2, pad 1 (max_pool_fallback, dabnn/layers/MaxPool.cpp:209-246), in one pass that never writes the
  * convolution's output: the stem of a Bi-Real-style net.  pooled [n][oh/2][ow/2][cout] receives what dab_max_pool
  * computes from the convolution's result; pooled_packed, when not null (cout % 64 == 0), pack_mat of it
- * (dabnn/bitpack.h:277-293) as dab_max_pool_sign writes it.  carry is a workspace of
- * dab_fconv_maxpool_carry_floats(...) floats.  Shapes: the convolution's output width ow must divide 448 into an even
+ * (dabnn/bitpack.h:277-293) as dab_max_pool_sign writes it (where a window's maximum is a zero of either sign, pooled
+ * may hold the zero of the other sign than dab_max_pool's: equal as numbers, and the same bit in pooled_packed).  carry is
+ * a workspace of dab_fconv_maxpool_carry_floats(...) floats, whose contents after the call are unspecified.  Shapes: the convolution's output width ow must divide 448 into an even
  * number of rows (28, 56, 112 or 224), oh must be a multiple of 448/ow, c must be 3 or a multiple of 4, cout a
  * multiple of 4, all buffers 16-byte aligned (DAB_EUNSUPPORTED otherwise).
  * dab_fconv_maxpool_carry_floats returns 0 for shapes the pass does not take; dab_fconv_maxpool_pays returns 1 when
