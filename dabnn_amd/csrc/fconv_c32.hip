@@ -175,21 +175,26 @@ __global__ __launch_bounds__(kC32Threads) void fconv_c32_kernel(const FconvC32Ar
     // {1, 2, 3} (v1): lane f (even) takes the maximum over pixels f - 1, f, f + 1 of the tile and stores pooled pixel f / 2
     auto pool_store = [&](const Place &at, int nt, int g_now, const f32x4w &v0, const f32x4w &v1) __attribute__((always_inline)) {
         const int lowest = __float_as_int(-FLT_MAX);
+        float h[2][4];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const f32x4w &v = half ? v1 : v0;
-            float h[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float left = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x111, 0xf, 0xf, false));
                 const float right = __int_as_float(__builtin_amdgcn_update_dpp(lowest, __float_as_int(v[e]), 0x101, 0xf, 0xf, false));
-                h[e] = max_of_three(left, v[e], right);
-            }
-            if (!(f_i & 1)) {
-                const size_t cell = ((size_t)at.img * (p.oh >> 1) + (at.oy0 >> 1) + half) * (p.ow >> 1) + at.xt * 8 + (f_i >> 1);
-                *reinterpret_cast<float4 *>(p.out + cell * COUT + nt * 16 + 4 * g_now) = make_float4(h[0], h[1], h[2], h[3]);
+                h[half][e] = max_of_three(left, v[e], right);
             }
         }
+        // one store for both rows: the odd lanes take the second row's cell from the even lane below them
+        float out[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float second = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(h[1][e]), 0x111, 0xf, 0xf, true));
+            out[e] = (f_i & 1) ? second : h[0][e];
+        }
+        const size_t cell = ((size_t)at.img * (p.oh >> 1) + (at.oy0 >> 1) + (f_i & 1)) * (p.ow >> 1) + at.xt * 8 + (f_i >> 1);
+        *reinterpret_cast<float4 *>(p.out + cell * COUT + nt * 16 + 4 * g_now) = make_float4(out[0], out[1], out[2], out[3]);
     };
     // Writes the item at `at`, whose sums are in acc (special: an infinity or a NaN among its pixels or in the filters).
     auto write_item = [&](const Place &at, bool special) __attribute__((always_inline)) {
