@@ -551,7 +551,7 @@ int fconv_c32_try(const float *x, int n, int h, int w, int c, const float *wgt, 
 bool fconv_c32_pool_takes(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h, int stride_w, int dil_h,
                           int dil_w, int cout, int oh, int ow) {
     return oh % 4 == 0 && fconv_c32_takes(n, h, w, c, kh, kw, pad_h, pad_w, stride_h, stride_w, dil_h, dil_w, cout, oh, ow) &&
-           (long long)n * (oh / 2) * (ow / 2) * (cout / 4) < (1ll << 32);
+           (long long)n * (oh / 2) * (ow / 2) * (cout / 4) < (1ll << 32) - 256;  // the completing pass counts cells in 32 bits
 }
 
 long long fconv_c32_pool_workspace_floats(int n, int oh, int ow, int cout) {

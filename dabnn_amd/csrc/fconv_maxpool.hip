@@ -88,6 +88,58 @@ struct BandOut {
     int img, band, row0, n0, ytile;
 };
 
+// Pooling down the rows of a staged band: a thread takes four channels of one pooled column; column(px, c4) gives a
+// function h(r), the maximum of row r's three columns 2*px-1 .. 2*px+1.  Pooled row q is max(h[2q-1], h[2q], h[2q+1]);
+// for q = 0 the row above the band is left out: row -1 of the image does not exist, and the last row of the band
+// above arrives through the carry, which is this band's h[R-1] -- or, when this block made the band above just before
+// (fold), it is in `keep`: a thread has the same columns and channels in every band.
+// ROWS: the band's rows when the kernel knows them (all loads of a column are then asked for at once).
+template <bool SIGN, int SLOTS, int ROWS, class Column>
+__device__ __forceinline__ void pool_band_rows(const FconvPoolArgs &p, const BandOut o, int tid, float4 (&keep)[SLOTS], bool fold,
+                                               bool write_carry, Column column) {
+#pragma unroll
+    for (int slot = 0; slot < SLOTS; ++slot) {
+        const int it = tid + slot * kBandThreads;
+        if (it >= p.pw * 16) break;
+        const int c4 = it & 15, px = it >> 4;
+        const int co = o.n0 + c4 * 4;
+        const auto h_of = column(px, c4);
+        const float4 lowest = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+        float4 prev = fold ? keep[slot] : lowest, even = lowest;
+        const int rows = ROWS ? ROWS : p.band_rows;
+        constexpr int kUnrollRows = ROWS > 0 ? ROWS : 1;
+#pragma unroll kUnrollRows
+        for (int r = 0; r < rows; ++r) {
+            const float4 h = h_of(r);
+            if (r & 1) {
+                const float4 m = max3(even, h, lowest);
+                if (co < p.cout) {
+                    const size_t pix = (size_t)(o.img * p.ph + ((o.row0 + r) >> 1)) * p.pw + px;
+                    *reinterpret_cast<float4 *>(p.pooled + pix * p.cout + co) = m;
+                    if constexpr (SIGN) {
+                        // cout % 64 == 0: the 16 lanes of a pixel are one row of lanes, all of them here
+                        const uint32_t nib = sign_nibble(m);
+                        uint32_t lo = c4 < 8 ? nib << (4 * c4) : 0u, hi = c4 >= 8 ? nib << (4 * (c4 - 8)) : 0u;
+                        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+                        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+                        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+                        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+                        if (c4 == 0) p.bits[pix * (p.cout >> 6) + o.ytile] = ((uint64_t)hi << 32) | lo;
+                    }
+                }
+            } else {
+                even = max3(prev, h, lowest);  // r == 0 without fold: prev is the lowest value, the row above is left out
+            }
+            prev = h;
+        }
+        keep[slot] = prev;
+        if (write_carry && co < p.cout) {
+            const float4 m = max3(prev, lowest, lowest);
+            *reinterpret_cast<float4 *>(p.carry + ((size_t)(o.img * p.bands + o.band) * p.pw + px) * p.cout + co) = m;
+        }
+    }
+}
+
 // A finished band (a wave's accumulators: 7 x 2 tiles of 16 pixels x 16 channels, wave (wm, wn) = pixels 112*wm ..,
 // channels 32*wn ..) goes through LDS to the pooled tensor, the carry and the sign bits.  All threads of the block
 // call it after a barrier that ended every other use of `stage`.
@@ -135,58 +187,18 @@ __device__ __forceinline__ void band_epilogue(const FconvPoolArgs &p, float *sta
         default: stage_all(T{}, T{}, T{}); break;
     }
     __syncthreads();
-
-    // Pooling: a thread takes four channels of one pooled column and walks down the band's rows.  h = the maximum
-    // of the row's three columns 2*px-1 .. 2*px+1 (the first pooled column has two; one is read twice).  Pooled
-    // row q is max(h[2q-1], h[2q], h[2q+1]); for q = 0 the row above the band is left out: row -1 of the image
-    // does not exist, and the last row of the band above arrives through the carry, which is this band's h[R-1] --
-    // or, when this block made the band above just before (fold), it is in `keep`: a thread has the same columns
-    // and channels in every band.
-#pragma unroll
-    for (int slot = 0; slot < SLOTS; ++slot) {
-        const int it = tid + slot * kBandThreads;
-        if (it >= p.pw * 16) break;
-        const int c4 = it & 15, px = it >> 4;
-        const int co = o.n0 + c4 * 4;
+    const int ow = ROWS ? kBandPixels / ROWS : p.ow;
+    // h of row r = the maximum of the row's three columns 2*px-1 .. 2*px+1 (the first pooled column has two; one is
+    // read twice)
+    pool_band_rows<SIGN, SLOTS, ROWS>(p, o, tid, keep, fold, write_carry, [&](int px, int c4) {
         const float *col0 = &stage[(px == 0 ? 0 : 2 * px - 1) * kStageStride + c4 * 4];
         const float *col1 = &stage[(2 * px) * kStageStride + c4 * 4];
-        const float4 lowest = make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
-        float4 prev = fold ? keep[slot] : lowest, even = lowest;
-        // ROWS: the band's rows when the kernel knows them (all loads of a column are then asked for at once)
-        const int rows = ROWS ? ROWS : p.band_rows, ow = ROWS ? kBandPixels / ROWS : p.ow;
-        constexpr int kUnrollRows = ROWS > 0 ? ROWS : 1;
-#pragma unroll kUnrollRows
-        for (int r = 0; r < rows; ++r) {
+        return [=](int r) {
             const int ro = r * ow * kStageStride;
-            const float4 h = max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
-                                  *reinterpret_cast<const float4 *>(col1 + ro + kStageStride));
-            if (r & 1) {
-                const float4 m = max3(even, h, lowest);
-                if (co < p.cout) {
-                    const size_t pix = (size_t)(o.img * p.ph + ((o.row0 + r) >> 1)) * p.pw + px;
-                    *reinterpret_cast<float4 *>(p.pooled + pix * p.cout + co) = m;
-                    if constexpr (SIGN) {
-                        // cout % 64 == 0: the 16 lanes of a pixel are one row of lanes, all of them here
-                        const uint32_t nib = sign_nibble(m);
-                        uint32_t lo = c4 < 8 ? nib << (4 * c4) : 0u, hi = c4 >= 8 ? nib << (4 * (c4 - 8)) : 0u;
-                        lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
-                        lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
-                        lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
-                        lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
-                        if (c4 == 0) p.bits[pix * (p.cout >> 6) + o.ytile] = ((uint64_t)hi << 32) | lo;
-                    }
-                }
-            } else {
-                even = max3(prev, h, lowest);  // r == 0 without fold: prev is the lowest value, the row above is left out
-            }
-            prev = h;
-        }
-        keep[slot] = prev;
-        if (write_carry && co < p.cout) {
-            const float4 m = max3(prev, lowest, lowest);
-            *reinterpret_cast<float4 *>(p.carry + ((size_t)(o.img * p.bands + o.band) * p.pw + px) * p.cout + co) = m;
-        }
-    }
+            return max3(*reinterpret_cast<const float4 *>(col0 + ro), *reinterpret_cast<const float4 *>(col1 + ro),
+                        *reinterpret_cast<const float4 *>(col1 + ro + kStageStride));
+        };
+    });
 }
 
 template <int CV, bool SIGN>
@@ -353,39 +365,107 @@ __global__ __launch_bounds__(kBandThreads) void fconv_maxpool_kernel(const Fconv
 //
 // The products run on the bf16 matrix cores with fp32 accuracy (split operands, six v_mfma_f32_16x16x32_bf16 per 32
 // depths; common.h): the instruction takes 19 cycles where the eight fp32 ones for the same depth take 256.  The tile
-// is split once, on its way into LDS, into three planes of bf16 (hi, mid, lo); the filters stay fp32 in LDS and are
-// split when a wave reads them, once per band and depth group.  The cross terms need hi with non-finite values taken
-// out (common.h); a band with an infinity or a NaN in its rows -- a flag in LDS says so -- takes a second copy of the
-// loop that derives it from hi in registers, all other bands use hi as it is.  A depth group is
+// is split once, on its way into LDS, into three planes of bf16 (hi, mid, lo), and so are the block's 64 filters, once
+// for all of its bands, in the order the instruction wants them (a lane's eight depths are 16 contiguous bytes).  The
+// cross terms need hi with non-finite values taken out (common.h); a band with an infinity or a NaN in its rows or in
+// the filters -- flags in LDS say so -- takes a second copy of the loop that derives it from hi in registers, all
+// other bands use hi as it is.  A depth group is
 // four slots of eight depths, slot g = lane / 16; the 147 depths make 19 slots: q = 0..13: kernel row q / 2, k' = 0..7
 // or 8..15; q = 14..17: k' = 16..19 of kernel rows (0, 1), (2, 3), (4, 5), (6, none); q = 18: k' = 20 of the seven
 // kernel rows, which a second small array per plane holds transposed (T20[ox][tile row]) so that they are contiguous
 // too; q = 19 is empty.  Empty halves read a zero area of the plane; the eighth element of slot 18 is masked (it is a
 // real tile value, and zero times an infinity would be a NaN).  160 depths for 147, five groups.
-// The block's 64 filters sit in LDS for all of its bands; the next band's rows are fetched into registers while the
-// current one is pooled.
+// The next band's rows are fetched into registers while the current one is pooled.  Pooling starts in registers: a
+// lane holds four neighbouring pixels of a row, so the maxima over the columns 2*px-1 .. 2*px+1 of two pooled columns
+// need one value from the lane 16 below; only those maxima -- half of the band -- are staged in LDS for the pass
+// down the rows.
 constexpr int kTileStride = 692;                    // elements per tile row: 115 pixel pairs x 6, + 2
 constexpr int kTileRows = 13, kTilePairs = 115;
 constexpr int kPlaneZero = 9000;                    // eight zeros behind the 13 x 692 tile elements
 constexpr int kPlaneT20 = kPlaneZero + 8;           // [112 output columns][16]: tile rows of element 6 * ox + 20
 constexpr int kPlane = kPlaneT20 + 112 * 16;        // bf16 elements per plane
-constexpr int kFilterStride = 148;                  // 7 x (16 + 4) + 7 + 1 floats per filter
-constexpr int kFilterFloats = kBandChannels * kFilterStride;
-constexpr int kStemLdsFloats = kFilterFloats + kBandPixels * kStageStride;  // the planes share the staged band's space
+constexpr int kStemDepth = 160;                     // 5 groups x 4 slots x 8
+constexpr int kFilterRow = kStemDepth + 8;          // bf16 elements per filter in a plane
+constexpr int kFilterPlane = kBandChannels * kFilterRow;
+constexpr int kStemStageStride = 72;                // floats per pooled column of the staged maxima: two columns on are 16 banks on
+constexpr int kStemStageFloats = 4 * 56 * kStemStageStride;
+constexpr int kStemWorkBytes = 3 * kPlane * 2 > kStemStageFloats * 4 ? 3 * kPlane * 2 : kStemStageFloats * 4;  // the planes share the staged maxima's space
 constexpr int kPairLoads = (kTileRows * kTilePairs + kBandThreads - 1) / kBandThreads;
 constexpr int kStemKeepSlots = 2;  // 56 pooled columns x 16 channel groups on 512 threads
 static_assert(56 * 16 <= kStemKeepSlots * kBandThreads, "pooled columns of the stem");
 static_assert(kTileStride * kTileRows <= kPlaneZero && (kPlaneT20 * 2) % 16 == 0 && (kPlane * 2) % 16 == 0, "plane layout");
-static_assert(3 * kPlane * 2 <= kBandPixels * kStageStride * 4, "the three planes fit the staged band's space");
+static_assert((kFilterRow * 2) % 16 == 0 && kStemWorkBytes % 16 == 0, "filter rows and the work area are 16-byte aligned");
+
+// The stem's finished band (accumulator element e of lane l: pixel 16*i + 4*(l/16) + e of row wm, channel l % 16 of
+// tile j): + bias, Affine (a*v + b, two roundings), Relu, in the reference's order; then the maxima over the columns
+// of the two pooled columns 8*i + 2*(l/16) and the next one go to LDS, and pool_band_rows walks down the four rows.
+// All threads of the block call it after a barrier that ended every other use of `stage`.
+template <bool SIGN>
+__device__ __forceinline__ void stem_epilogue(const FconvPoolArgs &p, float *stage, const f32x4v (&acc)[7][2], const BandOut o,
+                                              int tid, int wm, int wn, int f_s, int f_i, float4 (&keep)[kStemKeepSlots],
+                                              bool fold, bool write_carry) {
+    constexpr int TM = 7, TN = 2;
+    const int below = (((tid & 63) - 16) & 63) * 4;  // ds_bpermute address of the lane 16 below (lanes 0..15: 48 above)
+    auto stage_all = [&](auto has_bias, auto has_affine, auto has_relu) {
+#pragma clang fp contract(off)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int col = wn * (TN * 16) + j * 16 + f_i, co = o.n0 + col;
+            const bool co_ok = co < p.cout;
+            const float bias = (decltype(has_bias)::value && co_ok) ? p.bias[co] : 0.f;
+            const float fa = (decltype(has_affine)::value && co_ok) ? p.aff_a[co] : 0.f;
+            const float fb = (decltype(has_affine)::value && co_ok) ? p.aff_b[co] : 0.f;
+            float left = -FLT_MAX;  // lanes 0..15: the last pixel of the tile before (none before the first)
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = acc[i][j][e];
+                    if constexpr (decltype(has_bias)::value) v[e] = v[e] + bias;
+                    if constexpr (decltype(has_affine)::value) {
+                        const float prod = fa * v[e];
+                        v[e] = prod + fb;
+                    }
+                    if constexpr (decltype(has_relu)::value) v[e] = v[e] < 0.f ? 0.f : v[e];  // std::max(v, 0.f): a NaN stays
+                }
+                const float from_below = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(below, __builtin_bit_cast(int, v[3])));
+                const float before = f_s > 0 ? from_below : left;
+                left = from_below;
+                float *d = &stage[(wm * 56 + i * 8 + 2 * f_s) * kStemStageStride + col];
+                d[0] = max3(before, v[0], v[1]);
+                d[kStemStageStride] = max3(v[1], v[2], v[3]);
+            }
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    switch ((p.bias ? 4 : 0) | (p.aff_a ? 2 : 0) | (p.relu ? 1 : 0)) {
+        case 0: stage_all(F{}, F{}, F{}); break;
+        case 1: stage_all(F{}, F{}, T{}); break;
+        case 2: stage_all(F{}, T{}, F{}); break;
+        case 3: stage_all(F{}, T{}, T{}); break;
+        case 4: stage_all(T{}, F{}, F{}); break;
+        case 5: stage_all(T{}, F{}, T{}); break;
+        case 6: stage_all(T{}, T{}, F{}); break;
+        default: stage_all(T{}, T{}, T{}); break;
+    }
+    __syncthreads();
+    pool_band_rows<SIGN, kStemKeepSlots, 4>(p, o, tid, keep, fold, write_carry, [&](int px, int c4) {
+        const float *col = &stage[px * kStemStageStride + c4 * 4];
+        return [=](int r) { return *reinterpret_cast<const float4 *>(col + r * (56 * kStemStageStride)); };
+    });
+}
 
 template <bool SIGN>
 __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const FconvPoolArgs p) {
     constexpr int BN = kBandChannels, TM = 7, TN = 2;
     typedef uint32_t u32x2a __attribute__((ext_vector_type(2), aligned(4)));
-    __shared__ __attribute__((aligned(16))) float smem[kStemLdsFloats];
-    float *const wl = smem, *const stage = smem + kFilterFloats;
-    uint16_t *const planes = reinterpret_cast<uint16_t *>(stage);  // hi, mid, lo: kPlane elements each
-    __shared__ int special_flag;  // the band's rows hold an infinity or a NaN
+    __shared__ __attribute__((aligned(16))) uint16_t fplanes[3 * kFilterPlane];  // the filters: hi, mid, lo
+    __shared__ __attribute__((aligned(16))) float stage[kStemWorkBytes / 4];
+    uint16_t *const planes = reinterpret_cast<uint16_t *>(stage);  // the band's rows: hi, mid, lo, kPlane elements each
+    __shared__ int special_flag;    // the band's rows hold an infinity or a NaN
+    __shared__ int special_filters;  // 1 + the first channel of a channel tile whose filters hold one, or 0
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
@@ -442,27 +522,24 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         }
     };
 
-    // lane constants of the operand reads: the plane elements of a slot's two halves of four (tile i of the wave's
-    // row: + 96 * i; slot 18: + 256 * i; the zero area: + 0) and the floats of the same depths in a filter.  Groups
-    // 0..2 and the first two slots of group 3 are eight consecutive k' of kernel row 2 * G + g / 2: group 0's
-    // offsets plus a constant.  The other slots of group 3 and group 4 have offsets of their own.
+    // lane constants of the tile reads: the plane elements of a slot's two halves of four (tile i of the wave's
+    // row: + 96 * i; slot 18: + 256 * i; the zero area: + 0).  Groups 0..2 and the first two slots of group 3 are
+    // eight consecutive k' of kernel row 2 * G + g / 2: group 0's offsets plus a constant.  The other slots of group
+    // 3 and group 4 have offsets of their own.  (The filter planes are laid out slot by slot when they are filled.)
     const int base_a = 2 * wm * kTileStride + 6 * f_i;
-    const int a_main = base_a + (f_s >> 1) * kTileStride + 8 * (f_s & 1), b_main = (f_s >> 1) * 20 + 8 * (f_s & 1);
+    const int a_main = base_a + (f_s >> 1) * kTileStride + 8 * (f_s & 1);
     // group 3: slots 12, 13 (kernel row 6), 14, 15 (k' = 16..19 of kernel rows (0, 1) and (2, 3))
     const int a0_g3 = f_s < 2 ? a_main + 6 * kTileStride : base_a + 2 * (f_s - 2) * kTileStride + 16;
     const int a1_g3 = a0_g3 + (f_s < 2 ? 4 : kTileStride);
-    const int b0_g3 = f_s < 2 ? b_main + 120 : 2 * (f_s - 2) * 20 + 16, b1_g3 = b0_g3 + (f_s < 2 ? 4 : 20);
     // group 4: slots 16 (kernel rows 4, 5), 17 (row 6, nothing), 18 (k' = 20 of all rows), 19 (nothing)
     const int a0_g4 = f_s < 2 ? base_a + (4 + 2 * f_s) * kTileStride + 16 : f_s == 2 ? kPlaneT20 + f_i * 16 + 2 * wm : kPlaneZero;
     const int a1_g4 = f_s == 0 ? a0_g4 + kTileStride : f_s == 2 ? a0_g4 + 4 : kPlaneZero;
     const int s0_g4 = f_s < 2 ? 96 : f_s == 2 ? 256 : 0, s1_g4 = f_s == 0 ? 96 : f_s == 2 ? 256 : 0;
-    const int b0_g4 = f_s < 2 ? (4 + 2 * f_s) * 20 + 16 : f_s == 2 ? 140 : 0, b1_g4 = f_s == 0 ? b0_g4 + 20 : f_s == 2 ? 144 : 0;
-    const bool b0_ok_g4 = f_s != 3, b1_ok_g4 = f_s == 0 || f_s == 2;
     const uint32_t keep_g4 = f_s == 2 ? 0x0000ffffu : 0xffffffffu;  // slot 18: seven kernel rows, the eighth element out
 
     enter(item);
     fetch_tile();
-    if (tid == 0) special_flag = 0;
+    if (tid == 0) special_flag = 0, special_filters = 0;
     __syncthreads();
     int filters_of = -1;  // the channel tile whose filters are in LDS
     for (;;) {
@@ -470,12 +547,32 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         if (n0 != filters_of) {
             filters_of = n0;
             const int rows_n = p.cout - n0 < BN ? p.cout - n0 : BN;
-            for (int idx = tid; idx < kFilterFloats; idx += kBandThreads) {
-                const int co = idx / kFilterStride, r = idx - co * kFilterStride;
-                // r < 140: kernel row r / 20, k' = r % 20; then k' = 20 of kernel rows 0..6; the last float is zero
-                const int k = r < 140 ? (r / 20) * 21 + r % 20 : (r - 140) * 21 + 20;
-                wl[idx] = (co < rows_n && r < 147) ? p.w[(size_t)(n0 + co) * 147 + k] : 0.f;
+            bool special = false;
+            // two consecutive places of a filter's 160: slot q = place / 8, element t = place % 8
+            for (int idx = tid; idx < BN * (kStemDepth / 2); idx += kBandThreads) {
+                const int co = idx / (kStemDepth / 2), pr = idx - co * (kStemDepth / 2);
+                SplitParts sp[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const int q = (2 * pr + e) >> 3, t = (2 * pr + e) & 7;
+                    int k = -1;  // the place's depth in the filter's (kernel row, k') order
+                    if (q < 14) {
+                        k = (q >> 1) * 21 + 8 * (q & 1) + t;
+                    } else if (q < 18) {
+                        const int ky = 2 * (q - 14) + (t >> 2);
+                        if (ky < 7) k = ky * 21 + 16 + (t & 3);
+                    } else if (q == 18 && t < 7) {
+                        k = t * 21 + 20;
+                    }
+                    sp[e] = split_bf16x3((co < rows_n && k >= 0) ? p.w[(size_t)(n0 + co) * 147 + k] : 0.f);
+                    special |= sp[e].hif != sp[e].hi;
+                }
+                uint32_t *d = reinterpret_cast<uint32_t *>(fplanes + co * kFilterRow + 2 * pr);
+                d[0] = pack_upper_halves(sp[0].hi, sp[1].hi);
+                d[kFilterPlane / 2] = pack_upper_halves(sp[0].mid, sp[1].mid);
+                d[2 * (kFilterPlane / 2)] = pack_upper_halves(sp[0].lo, sp[1].lo);
             }
+            if (special) special_filters = n0 + 1;
         }
         if (tid < 12) reinterpret_cast<uint32_t *>(planes + (tid >> 2) * kPlane + kPlaneZero)[tid & 3] = 0u;
         bool any_special = false;
@@ -530,35 +627,54 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
             }
             return f;
         };
-        auto b_frag = [&](int j, int e0, int e1, bool ok0, bool ok1) {
-            const float *row = wl + (wn * 32 + j * 16 + f_i) * kFilterStride;
-            const float4 v0 = *reinterpret_cast<const float4 *>(row + e0), v1 = *reinterpret_cast<const float4 *>(row + e1);
-            const float x[8] = {ok0 ? v0.x : 0.f, ok0 ? v0.y : 0.f, ok0 ? v0.z : 0.f, ok0 ? v0.w : 0.f,
-                                ok1 ? v1.x : 0.f, ok1 ? v1.y : 0.f, ok1 ? v1.z : 0.f, ok1 ? v1.w : 0.f};
+        auto b_frag = [&](auto derive_finite, int G, int j) {
+            const uint16_t *row = fplanes + (wn * 32 + j * 16 + f_i) * kFilterRow + G * 32 + f_s * 8;
             SplitFrag8 f;
-            f.set(x);
+            f.hi = *reinterpret_cast<const SplitFrag8::u4 *>(row);
+            f.mid = *reinterpret_cast<const SplitFrag8::u4 *>(row + kFilterPlane);
+            f.lo = *reinterpret_cast<const SplitFrag8::u4 *>(row + 2 * kFilterPlane);
+            if constexpr (decltype(derive_finite)::value) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) f.hif[e] = finite_bf16_pair(f.hi[e]);
+            } else {
+                f.hif = f.hi;
+            }
             return f;
         };
+        auto tile_frag = [&](auto derive_finite, int G, int i) {
+            return G < 3    ? a_frag(derive_finite, a_main + 2 * G * kTileStride + 96 * i, a_main + 2 * G * kTileStride + 96 * i + 4, 0xffffffffu)
+                   : G == 3 ? a_frag(derive_finite, a0_g3 + 96 * i, a1_g3 + 96 * i, 0xffffffffu)
+                            : a_frag(derive_finite, a0_g4 + s0_g4 * i, a1_g4 + s1_g4 * i, keep_g4);
+        };
+        // 35 steps of twelve matrix instructions (depth group G = step / 7, pixel tile i = step % 7); a step's reads are
+        // the next step's tile fragment (six reads) and, in the middle of a group, the next group's filter fragments
+        // (six more), dealt out between its matrix instructions
         auto multiply = [&](auto derive_finite) {
+            SplitFrag8 a[2], b[2][TN];
 #pragma unroll
-            for (int G = 0; G < 5; ++G) {
-                SplitFrag8 b[TN];
+            for (int j = 0; j < TN; ++j) b[0][j] = b_frag(derive_finite, 0, j);
+            a[0] = tile_frag(derive_finite, 0, 0);
 #pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    b[j] = G < 3    ? b_frag(j, b_main + 40 * G, b_main + 40 * G + 4, true, true)
-                           : G == 3 ? b_frag(j, b0_g3, b1_g3, true, true)
-                                    : b_frag(j, b0_g4, b1_g4, b0_ok_g4, b1_ok_g4);
+            for (int step = 0; step < 5 * TM; ++step) {
+                const int G = step / TM, i = step - G * TM;
+                const bool more_tiles = step + 1 < 5 * TM, more_filters = i == 3 && G + 1 < 5;
+                if (more_tiles) a[(step + 1) & 1] = tile_frag(derive_finite, (step + 1) / TM, (step + 1) % TM);
+                if (more_filters) {
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const SplitFrag8 a =
-                        G < 3    ? a_frag(derive_finite, a_main + 2 * G * kTileStride + 96 * i, a_main + 2 * G * kTileStride + 96 * i + 4, 0xffffffffu)
-                        : G == 3 ? a_frag(derive_finite, a0_g3 + 96 * i, a1_g3 + 96 * i, 0xffffffffu)
-                                 : a_frag(derive_finite, a0_g4 + s0_g4 * i, a1_g4 + s1_g4 * i, keep_g4);
-                    mfma6_16x16x32(acc[i][0], acc[i][1], a, b[0], b[1]);
+                    for (int j = 0; j < TN; ++j) b[(G + 1) & 1][j] = b_frag(derive_finite, G + 1, j);
+                }
+                mfma6_16x16x32(acc[i][0], acc[i][1], a[step & 1], b[G & 1][0], b[G & 1][1]);
+                if constexpr (!decltype(derive_finite)::value) {
+#pragma unroll
+                    for (int k = 0; k < 6; ++k) {
+                        if (more_tiles) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // one LDS read
+                        if (more_filters) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // and one of the filters'
+                        __builtin_amdgcn_sched_group_barrier(0x8, 2, 0);                      // two matrix instructions
+                    }
                 }
             }
         };
-        if (__builtin_amdgcn_readfirstlane(special_flag) != 0)
+        if (__builtin_amdgcn_readfirstlane(special_flag) != 0 || __builtin_amdgcn_readfirstlane(special_filters) == n0 + 1)
             multiply(std::true_type{});
         else
             multiply(std::false_type{});
@@ -571,7 +687,7 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         }
         __syncthreads();  // the planes are dead: the staged band takes their place
         if (tid == 0) special_flag = 0;  // the next band's rows set it again, after the barrier that ends this pass
-        band_epilogue<SIGN, kStemKeepSlots, 4>(p, stage, acc, o, tid_band, wm, wn, f_s, f_i, keep, fold && o.band > 0, !p.chained || !has_next);
+        stem_epilogue<SIGN>(p, stage, acc, o, tid_band, wm, wn, f_s, f_i, keep, fold && o.band > 0, !p.chained || !has_next);
         if (!has_next) break;
         fold = p.chained != 0;
         item = next;
