@@ -580,21 +580,38 @@ __global__ __launch_bounds__(kBandThreads) void fconv7x7s2_maxpool_kernel(const 
         for (int j = 0; j < kPairLoads; ++j) {
             const PairPlace q = pair_place(j);
             if (q.lds >= 0) {
-                const SplitParts s[6] = {split_bf16x3(pf0[j][0]), split_bf16x3(pf0[j][1]), split_bf16x3(pf0[j][2]),
-                                         split_bf16x3(pf1[j][0]), split_bf16x3(pf1[j][1]), split_bf16x3(pf1[j][2])};
-                uint32_t *d = reinterpret_cast<uint32_t *>(planes + q.lds);
-#pragma unroll
-                for (int e = 0; e < 6; ++e) any_special |= s[e].hif != s[e].hi;
+                // the six values as three pairs through the packed conversions; a triple with an infinity, a NaN or a
+                // value that rounds up to an infinity is split again the slow way (and sends the band through the
+                // loop that derives the finite parts, which is right for finite values too)
+                const float v[6] = {pf0[j][0], pf0[j][1], pf0[j][2], pf1[j][0], pf1[j][1], pf1[j][2]};
+                SplitPair sp[3];
+                uint32_t magnitudes = 0;
 #pragma unroll
                 for (int e = 0; e < 3; ++e) {
-                    d[e] = pack_upper_halves(s[2 * e].hi, s[2 * e + 1].hi);
-                    d[kPlane / 2 + e] = pack_upper_halves(s[2 * e].mid, s[2 * e + 1].mid);
-                    d[2 * (kPlane / 2) + e] = pack_upper_halves(s[2 * e].lo, s[2 * e + 1].lo);
+                    sp[e] = split_pair_finite(v[2 * e], v[2 * e + 1]);
+                    magnitudes = bf16_pair_max(magnitudes, sp[e].hi);
                 }
-                if (q.t20 >= 0) {
-                    planes[q.t20] = (uint16_t)(s[2].hi >> 16);
-                    planes[kPlane + q.t20] = (uint16_t)(s[2].mid >> 16);
-                    planes[2 * kPlane + q.t20] = (uint16_t)(s[2].lo >> 16);
+                if (!bf16_pairs_finite(magnitudes)) {
+                    any_special = true;
+#pragma unroll
+                    for (int e = 0; e < 3; ++e) {
+                        const SplitParts s0 = split_bf16x3(v[2 * e]), s1 = split_bf16x3(v[2 * e + 1]);
+                        sp[e].hi = pack_upper_halves(s0.hi, s1.hi);
+                        sp[e].mid = pack_upper_halves(s0.mid, s1.mid);
+                        sp[e].lo = pack_upper_halves(s0.lo, s1.lo);
+                    }
+                }
+                uint32_t *d = reinterpret_cast<uint32_t *>(planes + q.lds);
+#pragma unroll
+                for (int e = 0; e < 3; ++e) {
+                    d[e] = sp[e].hi;
+                    d[kPlane / 2 + e] = sp[e].mid;
+                    d[2 * (kPlane / 2) + e] = sp[e].lo;
+                }
+                if (q.t20 >= 0) {  // the pair's third value: the first of the second pair
+                    planes[q.t20] = (uint16_t)sp[1].hi;
+                    planes[kPlane + q.t20] = (uint16_t)sp[1].mid;
+                    planes[2 * kPlane + q.t20] = (uint16_t)sp[1].lo;
                 }
             }
         }
