@@ -718,6 +718,27 @@ def test_fconv_maxpool_one_pass(dab, n, h, w, c, k, pad, stride, dil, cout, bias
     np.testing.assert_array_equal(pooled.cpu().numpy(), want)
     if sign:
         np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+    # the largest float in the image (its leading bf16 part would round up to an infinity) under filters of -1, 0, 1:
+    # every sum it takes part in is exact, and no window may turn infinite or NaN because of the split
+    xl = r.integers(-3, 4, x.shape).astype(np.float32)
+    xl[0, h // 2, w // 2, 0] = np.finfo(np.float32).max
+    xl[-1, h // 3, w // 3, c - 1] = -np.finfo(np.float32).max
+    wl = r.integers(-1, 2, wgt.shape).astype(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = cpu(xl, wl, bi, ai, ci)
+    pooled, packed = gpu(xl, wl, bi, ai, ci)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want)
+    # an infinite filter value: its channel is infinite where the tap meets a non-zero pixel and NaN where it meets a
+    # zero (padding included), as in the reference's product of the im2col matrix
+    xf = r.integers(-3, 4, x.shape).astype(np.float32)
+    wf = wi.copy()
+    wf[cout // 2, k // 2, 0, 0] = np.inf
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = cpu(xf, wf, bi, ai, ci)
+    pooled, packed = gpu(xf, wf, bi, ai, ci)
+    np.testing.assert_array_equal(pooled.cpu().numpy(), want)
+    if sign:
+        np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
 
 
 @pytest.mark.parametrize("n,h,w,pad,cout,bias,affine,relu", [
