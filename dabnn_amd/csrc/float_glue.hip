@@ -77,6 +77,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
     static_assert(TM >= 1 && TN >= 1 && WTM % 32 == 0 && WTN % 32 == 0, "wave tile");
     static_assert(WK % 8 == 0 && 256 % LK == 0 && APT >= 1 && BPT >= 1, "slice");
     static_assert(CV == 1 || CV == 4 || (CV == 3 && KSPLIT == 1), "channel-vector loader");
+    static_assert(KSPLIT == 1 || (KSPLIT == 4 && BM == 32 && BN == 32), "a split depth: the four waves share one 32 x 32 tile");
     static_assert(!POOL || (CV == 4 && !PADDED), "the pooling loader takes whole 2x2 windows of four channels");
     constexpr int NW = POOL ? 4 : 1;  // loads per tile element: the window of the pooled input
     constexpr bool B_PARTIAL = BN < RP;  // fewer weight rows than loader rows: the upper loader rows fetch nothing
@@ -631,6 +632,20 @@ int fill_f32(float *x, long long total, float v, hipStream_t s) {
 
 }  // namespace dab
 
+// 1x1 convolutions to 128 channels or more with fewer 128 x 128 tiles than CUs (the shortcut branches of a residual
+// net below batch 64 or so): the tile that still gives three quarters of the CUs a block -- 1: 64 x 128 with 32-deep
+// slices, 2: 64 x 64 with 32-deep slices, 3: 32 x 32 with 64-deep slices split over the four waves -- or 0 for other
+// shapes.  Measured inside a graph, AvePool 2x2 in the loader, against the 64 x 64 tiles with 16-deep slices that ran
+// before: 28 x 28 x 128 -> 256 at batch 64 / 32 / 16: 18.3 / 11.5 / 8.0 against 20.5 / 15.0 / 9.1 us; 14 x 14 x 256 ->
+// 512 at batch 64 / 32: 18.9 / 14.1 against 23.8 / 17.9.
+static int small_1x1_tiles(int taps, long long M, int cout) {
+    if (taps != 1 || cout < 128) return 0;
+    const long long want = 3ll * dab::simd_count() / 16;  // three quarters of the CUs
+    if (((M + 63) / 64) * ((cout + 127) / 128) >= want) return 1;
+    if (((M + 63) / 64) * ((cout + 63) / 64) >= want) return 2;
+    return 3;
+}
+
 static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
                       const float *aff_a, const float *aff_b, int relu, int kh, int kw, int pad_h, int pad_w, int stride_h,
                       int stride_w, int dil_h, int dil_w, int cout, float *out, dab_stream_t stream) {
@@ -693,6 +708,12 @@ static int fconv_impl(const char *fn, const float *x, int n, int h, int w, int c
         // a three-channel image too small for 128-pixel tiles (the stem at batch 1): 64-pixel tiles keep the
         // one-load-per-tap loader and still give most CUs a block
         DAB_FCONV_LAUNCH(64, 64, 24, 1, 3);
+    } else if (big_tiles < simd_count() / 4 && vec4 && small_1x1_tiles(kh * kw, M, cout) == 1) {
+        DAB_FCONV_LAUNCH(64, 128, 32, 1, 4);
+    } else if (big_tiles < simd_count() / 4 && vec4 && small_1x1_tiles(kh * kw, M, cout) == 2) {
+        DAB_FCONV_LAUNCH(64, 64, 32, 1, 4);
+    } else if (big_tiles < simd_count() / 4 && vec4 && small_1x1_tiles(kh * kw, M, cout) == 3) {
+        DAB_FCONV_LAUNCH(32, 32, 64, 4, 4);
     } else if (big_tiles < simd_count() / 4 && vec4 && ((M + 63) / 64) * ((cout + 63) / 64) >= simd_count() / 8) {
         // fewer big tiles than CUs, but enough 64 x 64 ones for half of them: a wave still multiplies a whole 32 x 32 tile
         DAB_FCONV_LAUNCH(64, 64, 16, 1, 4);
@@ -808,7 +829,15 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
 #define DAB_POOLED_LAUNCH(BM, BN, SK, KSPLIT)                                                                     \
     hipLaunchKernelGGL((fconv_kernel<BM, BN, SK, KSPLIT, false, 4, true>),                                        \
                        dim3((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN)), dim3(256), 0, s, a)
-    if (big_tiles < simd_count() / 4 && ((M + 63) / 64) * ((cout + 63) / 64) >= simd_count() / 8)
+    // the same tiles as dab_fconv_affine_relu takes for the 1x1 convolution of the pooled tensor: the sums of a tile
+    // whose depth is split over waves are added in another order
+    if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 1)
+        DAB_POOLED_LAUNCH(64, 128, 32, 1);
+    else if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 2)
+        DAB_POOLED_LAUNCH(64, 64, 32, 1);
+    else if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 3)
+        DAB_POOLED_LAUNCH(32, 32, 64, 4);
+    else if (big_tiles < simd_count() / 4 && ((M + 63) / 64) * ((cout + 63) / 64) >= simd_count() / 8)
         DAB_POOLED_LAUNCH(64, 64, 16, 1);
     else if (big_tiles < simd_count() / 4)
         DAB_POOLED_LAUNCH(32, 32, 64, 4);
