@@ -57,7 +57,11 @@ def main():
                          "calibrates the FETCH_SIZE / WRITE_SIZE counters.  headline (default): the same graph replay as "
                          "the timed region; fconv: the float convolutions of the Bi-Real-18 stems at batch 256, three "
                          "launches each, the two a MaxPool follows also as the one-pass kernel; bireal18: --steps runs "
-                         "of Bi-Real-18 (7x7 stem) at batch 256 through the C++ Net, layer by layer (no graph)")
+                         "of Bi-Real-18 (7x7 stem) at --profile-batch (256) through the C++ Net, layer by layer "
+                         "(eager launches, or the Net's graph replay with --profile-graph)")
+    ap.add_argument("--profile-batch", type=int, default=256, help="batch size of --profile-mode bireal18")
+    ap.add_argument("--profile-graph", action="store_true",
+                    help="--profile-mode bireal18: replay the Net's HIP graph (as an inference loop does) instead of eager launches")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no exchange between images, run it with --gpus 1 "
@@ -141,9 +145,9 @@ def main():
         from dabnn_amd import dab_format, models
         from dabnn_amd import net as dabnet
         mlayers, minits, minputs = models.bireal18(2024, stem=False)
-        net = dabnet.Net(batch=256).read_buf(dab_format.write_model(mlayers, minits, minputs))
-        net.set_use_graph(False)  # every layer a dispatch of its own, in layer order
-        x = torch.randn((256, 224, 224, 3), generator=g).cuda()
+        net = dabnet.Net(batch=args.profile_batch).read_buf(dab_format.write_model(mlayers, minits, minputs))
+        net.set_use_graph(args.profile_graph)  # without the graph every layer is a dispatch of its own, in layer order
+        x = torch.randn((args.profile_batch, 224, 224, 3), generator=g).cuda()
         for _ in range(max(1, args.warmup)):
             net.run(x)
         t_warm = time.perf_counter()
@@ -151,7 +155,8 @@ def main():
             net.run(x)
         for _ in range(args.steps):
             net.run(x)
-        print(json.dumps({"profile_mode": "bireal18", "batch": 256, "runs_after_warmup": args.steps,
+        print(json.dumps({"profile_mode": "bireal18", "batch": args.profile_batch, "graph": args.profile_graph,
+                          "runs_after_warmup": args.steps,
                           "layers": net.layers()}))
         net.close()
         return
