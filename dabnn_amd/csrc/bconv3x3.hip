@@ -398,6 +398,133 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
+// 56 x 56 x 64 -> 64 with Affine, Add and sign bits inside Bi-Real-18: batch 128 (24 tiles per CU) level with the unit
+// kernel, batch 64 behind it, batch 256 (49): 87-91 us a launch against 87-100, the net 1.619 against 1.631 ms
+constexpr int kTile64MinTilesPerCu = 32;
+
+// 64 input channels with an epilogue at large batch (the first stage of a residual net): the launch is bound by the
+// fp32 shortcut it reads and the fp32 result it writes, and the unit kernel's waves, each storing 8 KB windows of a
+// tile of its own, move them at 4.7-5.3 TB/s where a copy whose blocks take contiguous 16 KB chunks in turn reaches
+// 6.0.  Here a block's four waves share a tile of 64 pixels x 64 output channels: every wave counts 16 channels for
+// all 64 pixels (the tile's activations are 144 bytes per lane, fetched by each wave), the counts meet in LDS, and the
+// block reads the tile's shortcut, applies the epilogue and writes the result as one contiguous piece (256 bytes per
+// pixel; with more than 64 output channels a pixel's 64-channel part), 16 lanes to a pixel, so the sign bits of a
+// pixel are one row of lanes.  Tiles are dealt to the resident blocks in turn.
+constexpr int kTileRow = 64 * 4 + 16;  // bytes per pixel row of the staged tile: 16-byte writes of 16 lanes hit 64 banks once
+template <int MODE>
+__global__ __launch_bounds__(256) void bconv3x3_tile64_kernel(const BconvArgs p) {
+    static_assert(MODE == kModeAffineAdd || MODE == kModeAffineAddSign, "the tile kernel is for launches with an epilogue");
+    constexpr int K32 = 18, Q = 8;
+    __shared__ __attribute__((aligned(16))) unsigned char tile_lds[64 * kTileRow];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wib = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int column_tiles = p.cout >> 6;
+    const int tiles = (p.total + 63) >> 6;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
+    const int c4 = tid & 15;  // the thread's four channels of a pixel in the store pass
+
+    uint32_t a[K32];
+    auto fetch_tile = [&](int tile) {
+        {
+            int pix = tile * 64 + lane;
+            pix = pix < p.total ? pix : p.total - 1;
+            const uint32_t t = p.div_ow.div(pix);
+            const int ox = pix - t * p.OW;
+            const uint32_t n = p.div_oh.div(t);
+            const int oy = t - n * p.OH;
+            const int y0 = oy * p.stride - p.pad, x0 = ox * p.stride - p.pad;
+            const int base = ((n * p.H + y0) * p.W + x0) * 8;  // byte offset of tap (0,0); may be negative
+#pragma unroll
+            for (int kh = 0; kh < 3; ++kh) {
+                const bool row_ok = (unsigned)(y0 + kh) < (unsigned)p.H;
+#pragma unroll
+                for (int kw = 0; kw < 3; ++kw) {
+                    const bool ok = row_ok && (unsigned)(x0 + kw) < (unsigned)p.W;
+                    // an offset beyond the descriptor's range reads as zero: the reference's padding word
+                    const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, ok ? base + (kh * p.W + kw) * 8 : (int)0x80000000, 0, 0);
+                    a[(kh * 3 + kw) * 2] = v.x, a[(kh * 3 + kw) * 2 + 1] = v.y;
+                }
+            }
+        }
+    };
+    if ((int)blockIdx.x < tiles) fetch_tile((int)blockIdx.x);
+    for (int tile = (int)blockIdx.x; tile < tiles; tile += (int)gridDim.x) {
+        for (int ct = 0; ct < column_tiles; ++ct) {
+            // the store pass's shortcut values, asked for before the counting so that they arrive behind it:
+            // thread t has pixels t / 16 + 16 * j, j = 0..3, channels 4 * (t % 16) ..
+            const int pixel0 = tid >> 4;
+            const size_t out_off = ((size_t)tile * 64 + pixel0) * p.cout + ct * 64 + c4 * 4;
+            const size_t step = (size_t)16 * p.cout;  // 16 pixels on
+            float4 sc[4];
+            const bool with_shortcut = p.epi_shortcut != nullptr;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool ok = with_shortcut && tile * 64 + pixel0 + 16 * j < p.total;
+                sc[j] = ok ? *reinterpret_cast<const float4 *>(p.epi_shortcut + out_off + j * step) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            EpiAffineAdd epi;
+            epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+            epi.prepare(ct * 64 + c4 * 4);
+
+            // the wave's 16 channels of the lane's pixel
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                uint32_t acc[Q];
+                const int cg = ct * 8 + wib * 2 + u;  // group of eight output channels
+                unit_rowmajor<K32, Q>(p.w + (size_t)cg * Q * 9, a, acc);
+                float f[Q];
+#pragma unroll
+                for (int q = 0; q < Q; ++q) f[q] = __uint_as_float(acc[q]) - kAccBias;
+                unsigned char *row = tile_lds + lane * kTileRow + (wib * 16 + u * 8) * 4;
+                *reinterpret_cast<float4 *>(row) = make_float4(f[0], f[1], f[2], f[3]);
+                *reinterpret_cast<float4 *>(row + 16) = make_float4(f[4], f[5], f[6], f[7]);
+            }
+            // the tile's activations are dead: the next tile's come while this one is written
+            if (ct == column_tiles - 1 && tile + (int)gridDim.x < tiles) fetch_tile(tile + (int)gridDim.x);
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int pixel = pixel0 + 16 * j;
+                const float4 v = *reinterpret_cast<const float4 *>(tile_lds + pixel * kTileRow + c4 * 16);
+                const float4 r = with_shortcut ? epi.template apply<true>(v, sc[j]) : epi.template apply<false>(v, sc[j]);
+                const bool ok = tile * 64 + pixel < p.total;
+                if (ok) {
+                    typedef float f32x4 __attribute__((ext_vector_type(4)));
+                    __builtin_nontemporal_store(f32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<f32x4 *>(p.out + out_off + j * step));
+                }
+                if constexpr (MODE == kModeAffineAddSign) {
+                    // the 16 lanes of a pixel are one row of lanes
+                    const uint32_t nib = sign_nibble(r);
+                    uint32_t lo = c4 < 8 ? nib << (4 * c4) : 0u, hi = c4 >= 8 ? nib << (4 * (c4 - 8)) : 0u;
+                    lo = or_from_lane_above<1>(lo), hi = or_from_lane_above<1>(hi);
+                    lo = or_from_lane_above<2>(lo), hi = or_from_lane_above<2>(hi);
+                    lo = or_from_lane_above<4>(lo), hi = or_from_lane_above<4>(hi);
+                    lo = or_from_lane_above<8>(lo), hi = or_from_lane_above<8>(hi);
+                    if (ok && c4 == 0)
+                        *reinterpret_cast<uint64_t *>(p.epi_bits + ((size_t)tile * 64 + pixel) * (p.cout >> 3) + ct * 8) = ((uint64_t)hi << 32) | lo;
+                }
+            }
+            __syncthreads();  // the staged tile is dead
+        }
+    }
+}
+
+// Whether the tile kernel takes a launch: 64 input channels, an epilogue, whole 64-channel tiles of output, and enough
+// tiles that every resident block gets several (below that the unit kernel's finer split of the work is ahead).
+static bool takes_tile64(long long tiles, int cin, int cout, int mode) {
+    return cin == 64 && cout % 64 == 0 && (mode == kModeAffineAdd || mode == kModeAffineAddSign) &&
+           tiles >= kTile64MinTilesPerCu * (long long)(simd_count() / 4);
+}
+
+template <int MODE>
+static int launch_tile64(BconvArgs &a, long long tiles, hipStream_t stream) {
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_tile64_kernel<MODE>, 256);
+    const long long resident = (long long)(simd_count() / 4) * blocks_per_cu;
+    hipLaunchKernelGGL((bconv3x3_tile64_kernel<MODE>), dim3((unsigned)(tiles < resident ? tiles : resident)), dim3(256), 0, stream, a);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
 // Which kernel runs a problem of `tiles` 64-pixel tiles: 0 = the small-problem kernel (blocks split the depth),
 // 1 = the unit kernel at its wide residency, 2 = its second build: four waves per SIMD and whole-line stores for 64
 // and 128 input channels, units of twice the channels for 256 and 512.
@@ -418,6 +545,9 @@ static int pick_build(long long tiles, int cin, int cout) {
 
 template <int CW, int MODE>
 static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
+    if constexpr (CW == 1 && (MODE == kModeAffineAdd || MODE == kModeAffineAddSign)) {
+        if (takes_tile64(tiles, 64, a.cout, MODE)) return launch_tile64<MODE>(a, tiles, stream);
+    }
     const int build = pick_build(tiles, CW * 64, a.cout);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
     if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
@@ -521,6 +651,11 @@ extern "C" int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int
 extern "C" int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout) {
     if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return 0;
     return dab::splits_depth((n_out_pixels + 63) / 64, cin, cout) ? 1 : 0;
+}
+
+extern "C" int dab_bconv3x3_fused_shares_tiles(int64_t n_out_pixels, int cin, int cout) {
+    if (n_out_pixels <= 0 || cout <= 0) return 0;
+    return dab::takes_tile64((n_out_pixels + 63) / 64, cin, cout, dab::kModeAffineAdd) ? 1 : 0;
 }
 
 extern "C" int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout) {

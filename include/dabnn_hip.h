@@ -180,6 +180,14 @@ DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
 DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
 
 /*
+ * No counterpart in the reference: whether dab_bconv3x3_affine_add(_sign) runs a problem of n_out_pixels = N*OH*OW on
+ * the kernel whose blocks share a tile of 64 pixels x 64 output channels and write it as one piece (64 input channels,
+ * cout a multiple of 64, at least 32 tiles per CU: the first stage of a residual net at large batch, bound by the fp32
+ * shortcut it reads and the result it writes) instead of the build dab_bconv3x3_build names.  1 or 0.  For tests.
+ */
+DAB_API int dab_bconv3x3_fused_shares_tiles(int64_t n_out_pixels, int cin, int cout);
+
+/*
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in

@@ -343,6 +343,47 @@ def test_fused_epilogues_of_the_named_build(dab, n, h, w, cin, cout, stride, bui
         np.testing.assert_array_equal(host_u(packed[i]), orc.pack_mat(want))
 
 
+@pytest.mark.parametrize("n,h,w,cout,stride", [
+    (168, 56, 56, 64, 1),    # a stage-1 block of Bi-Real-18 at batch 168: 8232 tiles
+    (180, 55, 55, 64, 1),    # a last tile that is not full
+    (170, 112, 112, 128, 2),  # two 64-channel tiles per pixel, stride 2
+])
+def test_fused_epilogues_of_the_shared_tile_kernel(dab, n, h, w, cout, stride):
+    """BinConv + Affine + Add (+ sign) over 64 input channels at a batch where a block's waves share a tile (asked
+    from the library): bit for bit the unit kernel's result on the two halves of the batch, which are below the
+    switch; three images against the three reference layers."""
+    from dabnn_amd import capi
+    oh = (h + 2 - 3) // stride + 1
+    assert capi.lib.dab_bconv3x3_fused_shares_tiles(n * oh * oh, 64, cout) == 1
+    assert capi.lib.dab_bconv3x3_fused_shares_tiles((n // 2 + 1) * oh * oh, 64, cout) == 0
+    r = rng(27)
+    x = r.integers(0, 2**64, size=(n, h, w, 1), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9), dtype=np.uint64)
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    a[::5] = 0.0
+    sc = r.standard_normal((n, oh, oh, cout)).astype(np.float32)
+    sc[:, :, :, ::10] = 0.0
+    xd, wd, ad, bd, scd = dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), dev_f(sc)
+    got1 = dab.bconv_3x3_affine_add(xd, wd, ad, bd, scd, stride, 1)
+    got2, packed = dab.bconv_3x3_affine_add_sign(xd, wd, ad, bd, scd, stride, 1)
+    nosc = dab.bconv_3x3_affine_add(xd, wd, ad, bd, None, stride, 1)
+    half = n // 2
+    for lo, hi in ((0, half), (half, n)):
+        want, want_bits = dab.bconv_3x3_affine_add_sign(xd[lo:hi].contiguous(), wd, ad, bd, scd[lo:hi].contiguous(), stride, 1)
+        assert torch.equal(got1[lo:hi], want)
+        assert torch.equal(got2[lo:hi], want)
+        assert torch.equal(packed[lo:hi], want_bits)
+        assert torch.equal(nosc[lo:hi], dab.bconv_3x3_affine_add(xd[lo:hi].contiguous(), wd, ad, bd, None, stride, 1))
+    for i in (0, half - 1, n - 1):
+        want = orc.baseline_bconv(x[i], wgt, 3, 3, 1, 1, stride, stride)
+        orc.affine_inplace(want, a, b)
+        np.testing.assert_array_equal(nosc[i].cpu().numpy(), want)
+        want = want + sc[i]
+        np.testing.assert_array_equal(got2[i].cpu().numpy(), want)
+        np.testing.assert_array_equal(host_u(packed[i]), orc.pack_mat(want))
+
+
 def test_bconv_3x3_unsupported_and_invalid(dab):
     from dabnn_amd.capi import DabUnsupported
     x = torch.zeros((1, 4, 4, 3), dtype=torch.int64, device="cuda")  # 192 channels
