@@ -412,7 +412,7 @@ constexpr int kTile64MinTilesPerCu = 32;
 // pixel are one row of lanes.  Tiles are dealt to the resident blocks in turn.
 constexpr int kTileRow = 64 * 4 + 16;  // bytes per pixel row of the staged tile: 16-byte writes of 16 lanes hit 64 banks once
 template <int MODE>
-__global__ __launch_bounds__(256) void bconv3x3_tile64_kernel(const BconvArgs p) {
+__global__ __launch_bounds__(256, 6) void bconv3x3_tile64_kernel(const BconvArgs p) {
     static_assert(MODE == kModeAffineAdd || MODE == kModeAffineAddSign, "the tile kernel is for launches with an epilogue");
     constexpr int K32 = 18, Q = 8;
     __shared__ __attribute__((aligned(16))) unsigned char tile_lds[64 * kTileRow];
@@ -466,8 +466,9 @@ __global__ __launch_bounds__(256) void bconv3x3_tile64_kernel(const BconvArgs p)
             epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
             epi.prepare(ct * 64 + c4 * 4);
 
-            // the wave's 16 channels of the lane's pixel
-#pragma unroll
+            // the wave's 16 channels of the lane's pixel, eight at a time (unrolled, the two units' registers keep the
+            // kernel from six waves per SIMD)
+#pragma unroll 1
             for (int u = 0; u < 2; ++u) {
                 uint32_t acc[Q];
                 const int cg = ct * 8 + wib * 2 + u;  // group of eight output channels
