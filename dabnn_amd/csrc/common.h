@@ -8,7 +8,7 @@
 #include <string>
 #include <utility>
 
-#include "../../include/dabnn_hip.h"
+#include "../../include/dabnn_hip_tuning.h"
 
 namespace dab {
 
@@ -105,9 +105,15 @@ __device__ __forceinline__ uint32_t or_from_lane_above(uint32_t v) {
 // cycles, six of them for 16 depths: 404 TFLOP/s fp32-equivalent against 156; v_mfma_f32_16x16x32_bf16 in 16-19 for
 // 32 depths; the splitting runs on the vector pipe while another wave's matrix instructions are in flight).
 // An infinity or a NaN stays whole in hi and takes part in the hi*hi term only, where it meets the other operand's
-// leading part -- the same sign and zero only where the operand is -- so x*w is infinite or NaN exactly where the
-// fp32 product is; the cross terms use `hif`, hi with non-finite values replaced by zero (an infinity times a zero
-// mid or lo part would be a NaN).  A NaN keeps a quiet bit in its upper half.
+// leading part -- the same sign, and zero where the operand is zero -- so x*w is infinite or NaN where the fp32
+// product is, as long as the other operand's leading part is a normal bf16 or an exact zero; the cross terms use
+// `hif`, hi with non-finite values replaced by zero (an infinity times a zero mid or lo part would be a NaN).  A NaN
+// keeps a quiet bit in its upper half.
+// Limits: the leading part of a nonzero |w| below 2^-126 (an fp32 denormal) is zero or a bf16 denormal, which the
+// matrix core may flush, so inf * w can come out as NaN or 0 where fp32 arithmetic gives an infinity; and for finite
+// operands within 2^16 of the smallest normal the mid and lo parts are bf16 denormals, so the fp32-equivalent error
+// bound above holds only for magnitudes of 2^-110 and more.  Float weights and activations of that size do not occur
+// in the networks this path serves, and no fixture of the reference covers them.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4w __attribute__((ext_vector_type(4)));
 

@@ -230,6 +230,7 @@ __device__ __forceinline__ void stage_put(unsigned char *stage, int lane, int ch
 //                     (pack_mat, dabnn/bitpack.h:277-293)
 struct EpiStore {
     static constexpr bool kEmit = false;
+    static constexpr bool kReadsOut = false;
     static constexpr bool kShortcut = false;  // the epilogue never reads a second tensor
     const float *shortcut = nullptr;
     __device__ __forceinline__ void prepare(int) {}
@@ -240,6 +241,7 @@ struct EpiStore {
 };
 struct EpiAffineAdd {
     static constexpr bool kEmit = false;
+    static constexpr bool kReadsOut = false;  // the shortcut is a tensor of its own
     static constexpr bool kShortcut = true;
     const float *a;
     const float *b;
@@ -263,8 +265,9 @@ struct EpiAffineAdd {
 // integers far below 2^24, their float sum is exact)
 struct EpiAccumulate {
     static constexpr bool kEmit = false;
+    static constexpr bool kReadsOut = true;  // the second operand is what `out` holds: read through `out` itself
     static constexpr bool kShortcut = true;
-    const float *shortcut;  // = out
+    const float *shortcut;  // non-null marker only; the store pass reads through its own `out` pointer
     __device__ __forceinline__ void prepare(int) {}
     template <bool SC>
     __device__ __forceinline__ float4 apply(float4 v, float4 sc) const {
@@ -297,7 +300,9 @@ __device__ __forceinline__ void stage_flush_window(const unsigned char *stage, i
         float4 sc[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-            if constexpr (SC)
+            if constexpr (SC && Epi::kReadsOut)
+                sc[g] = *reinterpret_cast<const float4 *>(out + off0 + (size_t)(i0 + g) * PPI * ld);
+            else if constexpr (SC)
                 sc[g] = *reinterpret_cast<const float4 *>(epi.shortcut + off0 + (size_t)(i0 + g) * PPI * ld);
             else
                 sc[g] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -359,7 +364,8 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
                 epi.prepare(cbase + part * 4);
                 float4 r;
                 if (has_sc)
-                    r = epi.template apply<Epi::kShortcut>(v, *reinterpret_cast<const float4 *>(epi.shortcut + off));
+                    r = epi.template apply<Epi::kShortcut>(
+                        v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
                 else
                     r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
                 *reinterpret_cast<float4 *>(out + off) = r;

@@ -3,7 +3,7 @@
 #include <sstream>
 #include <stdexcept>
 
-#include "../../include/dabnn_hip.h"
+#include "../../include/dabnn_hip_tuning.h"
 #include "net.h"
 
 namespace bnn {
@@ -12,6 +12,19 @@ void bnn_fail(const std::string &msg) { throw std::runtime_error(msg); }
 
 void dab_check(int rc) {
     if (rc != DAB_OK) throw std::runtime_error(dab_last_error());
+}
+
+// The kernels write n * oh * ow * c elements computed from the input and the window: the output blob a layer was
+// handed must have exactly that geometry (a blob of another layer under the same name would be smaller).
+static void check_window_output(const char *layer, const Mat &in, const Mat &out, int kh, int kw, int pad_h, int pad_w,
+                                int stride_h, int stride_w, int dil_h, int dil_w, int channels) {
+    BNN_ASSERT(stride_h > 0 && stride_w > 0 && pad_h >= 0 && pad_w >= 0 && kh > 0 && kw > 0, std::string(layer) + ": bad window");
+    const long long oh = ((long long)in.h + 2ll * pad_h - ((long long)dil_h * (kh - 1) + 1)) / stride_h + 1;
+    const long long ow = ((long long)in.w + 2ll * pad_w - ((long long)dil_w * (kw - 1) + 1)) / stride_w + 1;
+    BNN_ASSERT(out.data_type == DataType::Float && out.n == in.n && out.h == oh && out.w == ow && out.c == channels,
+               std::string(layer) + " output blob " + out.name + " is " + std::to_string(out.n) + "x" + std::to_string(out.h) + "x" +
+                   std::to_string(out.w) + "x" + std::to_string(out.c) + ", the layer makes " + std::to_string(in.n) + "x" +
+                   std::to_string(oh) + "x" + std::to_string(ow) + "x" + std::to_string(channels));
 }
 
 // ---------------------------------------------------------------- Layer
@@ -60,11 +73,17 @@ BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad
                                                                         std::to_string(9 * (input_mat->elem_c / 64)));
     }
 
+    check_window_output("BinConv", *input_mat, *output_mat, kernel_h(), kernel_w(), pad_h, pad_w, stride_h, stride_w, 1, 1,
+                        weight_mat->n);
+
     const std::string binarized_name = "binaized_for_" + output + "_cal";
     if (!n->has_blob(binarized_name))
         n->add_mat(binarized_name, std::make_shared<Mat>(input_mat->n, input_mat->h, input_mat->w, input_mat->elem_c,
                                                          DataType::Bit, binarized_name));
     binarized_mat = mat(binarized_name);
+    BNN_ASSERT(binarized_mat->data_type == DataType::Bit &&
+                   binarized_mat->total() >= (size_t)input_mat->n * input_mat->h * input_mat->w * (input_mat->elem_c / 64),
+               "blob " + binarized_name + " is too small for the packed input");
 
     const std::string col_name = "col_for_" + output + "_cal";
     if (!n->has_blob(col_name)) {
@@ -73,6 +92,10 @@ BinConv::BinConv(NetCP net, css name, css input, css weight, css output, int pad
         n->add_mat(col_name, std::make_shared<Mat>(len, DataType::Bit, col_name));
     }
     col_mat = mat(col_name);
+    BNN_ASSERT(col_mat->data_type == DataType::Bit &&
+                   col_mat->total() >= (size_t)output_mat->n * output_mat->h * output_mat->w *
+                                           dab_col_row_words(kernel_h(), kernel_w(), input_mat->elem_c),
+               "blob " + col_name + " is too small for the column matrix");
 
     const int m = weight_mat->n;
     const int k = (int)(weight_mat->total() / m);
@@ -189,6 +212,8 @@ void FloatConv::check_operands() const {
     BNN_ASSERT(output_mat->c == weight_mat->n, "FloatConv output does not have one channel per filter");
     if (bias_mat) BNN_ASSERT((int)bias_mat->total() == weight_mat->n, "FloatConv bias does not match the filter count");
     BNN_ASSERT(stride_h > 0 && stride_w > 0 && dilation > 0 && pad_h >= 0 && pad_w >= 0, "FloatConv: bad stride, dilation or pad");
+    check_window_output("FloatConv", *input_mat, *output_mat, weight_mat->h, weight_mat->w, pad_h, pad_w, stride_h, stride_w,
+                        dilation, dilation, weight_mat->n);
 }
 
 void FloatConv::forward_impl() const {
@@ -326,7 +351,10 @@ AvePool::AvePool(NetCP net, css name, css input, css output, int kernel_h_, int 
       pad_h(pad_h_),
       pad_w(pad_w_),
       stride_h(stride_h_),
-      stride_w(stride_w_) {}
+      stride_w(stride_w_) {
+    BNN_ASSERT(input_mat->data_type == DataType::Float, "pooling input must be float");
+    check_window_output("AvePool", *input_mat, *output_mat, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, 1, 1, input_mat->c);
+}
 
 void AvePool::forward_impl() const {
     dab_check(dab_ave_pool(static_cast<const float *>(input_mat->dev), input_mat->n, input_mat->h, input_mat->w,
@@ -344,7 +372,10 @@ MaxPool::MaxPool(NetCP net, css name, css input, css output, int kernel_h_, int 
       pad_h(pad_h_),
       pad_w(pad_w_),
       stride_h(stride_h_),
-      stride_w(stride_w_) {}
+      stride_w(stride_w_) {
+    BNN_ASSERT(input_mat->data_type == DataType::Float, "pooling input must be float");
+    check_window_output("MaxPool", *input_mat, *output_mat, kernel_h, kernel_w, pad_h, pad_w, stride_h, stride_w, 1, 1, input_mat->c);
+}
 
 void MaxPool::forward_impl() const {
     if (fused_sign_out) {

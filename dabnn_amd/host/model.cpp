@@ -1,5 +1,6 @@
 #include "model.h"
 
+#include <set>
 #include <sstream>
 #include <stdexcept>
 
@@ -222,11 +223,25 @@ void check_model(ModelDesc &m, bool run_fconv) {
         }
         return *it->second;
     };
-    auto set_out = [&](const std::string &n, uint32_t h, uint32_t w, uint32_t c, bool bit) {
+    // A layer that makes a new blob must not name it like the input, an initializer, an earlier output or one of the
+    // scratch blobs a BinConv registers: Net::prepare would keep the blob that exists, of another size, and the
+    // layer's kernel would write its own geometry into it.
+    std::set<std::string> scratch_names;
+    auto fresh_name = [&](const std::string &n, const std::string &layer) {
+        require(m.shapes.find(n) == m.shapes.end() && scratch_names.find(n) == scratch_names.end(),
+                "layer " + layer + ": output " + n + " names a blob that already exists");
+    };
+    auto set_out = [&](const std::string &n, uint32_t h, uint32_t w, uint32_t c, bool bit, const std::string &layer) {
+        fresh_name(n, layer);
+        // the element count of one image and of the output row index must fit the int fields of Mat and the kernels
+        require((uint64_t)h * w * c < (1ull << 31), "layer " + layer + ": output " + n + " is too large");
         m.shapes[n] = {1, h, w, c};
         m.is_bit[n] = bit;
     };
     auto alias = [&](const std::string &out, const std::string &in) {  // ADD_INPLACE_LAYER
+        // a second name for the input's blob; re-pointing an existing name (the net's input, say) at another blob
+        // would hand its earlier users' sizes to a blob of another size
+        if (out != in) fresh_name(out, "(in place) " + in);
         const auto s = shape_of(in);
         const bool bit = m.is_bit[in];
         m.shapes[out] = s;
@@ -256,6 +271,8 @@ void check_model(ModelDesc &m, bool run_fconv) {
                 require(!m.is_bit[l.inputs[0]], l.type == kBinConv2D ? "BinConv input must be float" : "FloatConv input must be float");
                 require(ws[3] == is[3], "layer " + l.name + ": weight " + l.weight + " has " + std::to_string(ws[3]) +
                                             " input channels, the input blob " + std::to_string(is[3]));
+                require(ws[1] <= (1u << 15) && ws[2] <= (1u << 15), "layer " + l.name + ": kernel " + std::to_string(ws[1]) + "x" +
+                                                                        std::to_string(ws[2]) + " is too large");
                 const uint32_t oh = window_out(is[1], l.pad_h, (int)ws[1], l.dil_h, l.stride_h, l.name);
                 const uint32_t ow = window_out(is[2], l.pad_w, (int)ws[2], l.dil_w, l.stride_w, l.name);
                 if (l.type == kBinConv2D) {
@@ -273,7 +290,19 @@ void check_model(ModelDesc &m, bool run_fconv) {
                     require(l.dil_h == l.dil_w, "FloatConv needs equal dilations");
                 }
                 if (!l.bias.empty()) float_vec(l.bias, ws[0], l.name, "bias");
-                set_out(l.outputs[0], oh, ow, ws[0], false);
+                set_out(l.outputs[0], oh, ow, ws[0], false, l.name);
+                if (l.type == kBinConv2D) {
+                    // the scratch blobs the layer registers under the reference's names (dabnn/layers/BinConv.cpp:17-57)
+                    for (const char *prefix : {"binaized_for_", "col_for_"}) {
+                        const std::string scratch = prefix + l.outputs[0] + "_cal";
+                        fresh_name(scratch, l.name);
+                        scratch_names.insert(scratch);
+                    }
+                    // the transposed weights are registered too; two layers may share a weight
+                    require(m.shapes.find("trans_" + l.weight) == m.shapes.end(),
+                            "layer " + l.name + ": trans_" + l.weight + " names a blob that already exists");
+                    scratch_names.insert("trans_" + l.weight);
+                }
                 (void)run_fconv;  // a skipped float convolution still defines its output blob (dabnn/net.cpp:145-170)
                 break;
             }
@@ -315,7 +344,8 @@ void check_model(ModelDesc &m, bool run_fconv) {
                 require(!m.is_bit[l.inputs[0]], "pooling input must be float");
                 const uint32_t oh = window_out(is[1], l.pad_h, l.kernel_shape[0], 1, l.stride_h, l.name);  // common/Shaper.cpp:127-145
                 const uint32_t ow = window_out(is[2], l.pad_w, l.kernel_shape[1], 1, l.stride_w, l.name);
-                set_out(l.outputs[0], oh, ow, is[3], false);
+                require(l.kernel_shape[0] <= (1 << 15) && l.kernel_shape[1] <= (1 << 15), "layer " + l.name + ": pooling window is too large");
+                set_out(l.outputs[0], oh, ow, is[3], false, l.name);
                 break;
             }
             case kConcat: {  // dabnn/net.cpp:230-236: two inputs, channel axis; shape as common/Shaper.cpp:157-178
@@ -325,7 +355,7 @@ void check_model(ModelDesc &m, bool run_fconv) {
                 const auto &s2 = blob4(l.inputs[1], l.name);
                 require(s1[1] == s2[1] && s1[2] == s2[2], "Wrong input for concat");
                 require(!m.is_bit[l.inputs[0]] && !m.is_bit[l.inputs[1]], "Concat inputs must be float");
-                set_out(l.outputs[0], s1[1], s1[2], s1[3] + s2[3], false);
+                set_out(l.outputs[0], s1[1], s1[2], s1[3] + s2[3], false, l.name);
                 break;
             }
             case kSplit: {  // dabnn/net.cpp:245-250, dabnn/layers/Split.h:16-24; shape as common/Shaper.cpp:245-260
@@ -334,6 +364,7 @@ void check_model(ModelDesc &m, bool run_fconv) {
                 require(m.is_bit[l.inputs[0]], "Split only supports bit mat");
                 require(s[3] % 128 == 0 && s[3] <= 512, "Split: " + std::to_string(s[3]) + " channels");
                 for (const std::string &o : l.outputs) {
+                    fresh_name(o, l.name);
                     m.shapes[o] = {s[0], s[1], s[2], s[3] / 2};
                     m.is_bit[o] = true;
                 }

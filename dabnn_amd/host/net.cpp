@@ -8,7 +8,7 @@
 #include <sstream>
 #include <stdexcept>
 
-#include "../../include/dabnn_hip.h"
+#include "../../include/dabnn_hip_tuning.h"
 #include "layers.h"
 #include "model.h"
 
@@ -122,6 +122,12 @@ void Net::prepare(const void *buf, size_t len) {
     ModelDesc model = parse_model(buf, len);
     check_model(model, run_fconv);
     for (const auto &kv : model.shapes) shapes_[kv.first] = kv.second;
+    // every blob of the batch must stay within the int extents of Mat and of the kernels' pixel counts
+    for (const auto &kv : model.shapes) {
+        if (kv.second.size() != 4) continue;
+        const uint64_t per_image = (uint64_t)kv.second[1] * kv.second[2] * kv.second[3];
+        BNN_ASSERT(per_image * (uint64_t)batch_ < (1ull << 31), "blob " + kv.first + " is too large at batch " + std::to_string(batch_));
+    }
 
     // inputs: the first one only (dabnn/net.cpp:59-70)
     {

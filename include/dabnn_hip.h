@@ -162,32 +162,6 @@ DAB_API int dab_bconv3x3_affine_add_sign(const uint64_t *x, int n, int h, int w,
                                          float *out, uint64_t *out_packed, dab_stream_t stream);
 
 /*
- * No counterpart in the reference: 1 when dab_bconv3x3* would run this problem (n_out_pixels = N*OH*OW) with its
- * small-problem kernel, whose work items are whole bytes of sign bits -- dab_bconv3x3_affine_add_sign then costs no
- * more than dab_bconv3x3_affine_add, also for 512 input channels (cin 64, 128, 256 or 512; other values answer 0), where the large kernel makes the packed copy
- * dearer than a separate dab_bitpack_nhwc.  0 otherwise.  Net::prepare uses it to decide which layers to link.
- */
-DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
-
-/*
- * No counterpart in the reference: which of the three builds of the direct kernel dab_bconv3x3* runs for a problem of
- * n_out_pixels = N*OH*OW on the current device: 0 = the small-problem kernel (a block splits the depth over its
- * waves), 1 = the unit kernel's build for mid-sized problems, 2 = its build for large ones (four waves per SIMD and
- * whole-line stores for 64 and 128 input channels, units of twice the channels for 256 and 512; taken when a wave
- * gets many units); -1 for shapes the direct kernel does not take.  For tests and tuning: a parity test names the
- * build it means to cover.
- */
-DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
-
-/*
- * No counterpart in the reference: whether dab_bconv3x3_affine_add(_sign) runs a problem of n_out_pixels = N*OH*OW on
- * the kernel whose blocks share a tile of 64 pixels x 64 output channels and write it as one piece (64 input channels,
- * cout a multiple of 64, at least 32 tiles per CU: the first stage of a residual net at large batch, bound by the fp32
- * shortcut it reads and the result it writes) instead of the build dab_bconv3x3_build names.  1 or 0.  For tests.
- */
-DAB_API int dab_bconv3x3_fused_shares_tiles(int64_t n_out_pixels, int cin, int cout);
-
-/*
  * BinConv::forward_impl (dabnn/layers/BinConv.cpp:144-191) for a batch of
  * fp32 NHWC images: binarise + binary convolution, fp32 mismatch counts out.
  * Method selection mirrors BinConv::method() (:80-98): 3x3 with cin in
@@ -258,14 +232,13 @@ DAB_API int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, c
  * FpConv2D (dabnn/fconv.h:14-76) and the optional Affine and Relu of dab_fconv_affine_relu, in one launch: the end of
  * a classifier at small batch.  pooled [n][1][1][c] receives the pooled tensor exactly as dab_ave_pool writes it, out
  * [n][1][1][cout] the convolution of it exactly as dab_fconv_affine_relu computes it from that tensor.  wgt is
- * [cout][1][1][c].  dab_global_ave_pool_fconv1x1_takes returns 1 for the shapes the launch covers (n <= 8,
+ * [cout][1][1][c].  dab_global_ave_pool_fconv1x1_takes (dabnn_hip_tuning.h) returns 1 for the shapes the launch covers (n <= 8,
  * h * w <= 64, c a multiple of 4 up to 1024, cout >= 64); others, and x, wgt or pooled not 16-byte aligned, are
  * DAB_EUNSUPPORTED: the two separate calls serve them.
  */
 DAB_API int dab_global_ave_pool_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
                                          const float *a, const float *b, int relu, int cout, float *pooled, float *out,
                                          dab_stream_t stream);
-DAB_API int dab_global_ave_pool_fconv1x1_takes(int n, int h, int w, int c, int cout);
 
 /*
  * FpConv2D (dabnn/fconv.h:14-76) with the optional Affine and Relu of dab_fconv_affine_relu, followed by MaxPool 3x3,
@@ -277,7 +250,7 @@ DAB_API int dab_global_ave_pool_fconv1x1_takes(int n, int h, int w, int c, int c
  * a workspace of dab_fconv_maxpool_carry_floats(...) floats, whose contents after the call are unspecified.  Shapes: the convolution's output width ow must divide 448 into an even
  * number of rows (28, 56, 112 or 224), oh must be a multiple of 448/ow, c must be 3 or a multiple of 4, cout a
  * multiple of 4, all buffers 16-byte aligned (DAB_EUNSUPPORTED otherwise).
- * dab_fconv_maxpool_carry_floats returns 0 for shapes the pass does not take; dab_fconv_maxpool_pays returns 1 when
+ * dab_fconv_maxpool_carry_floats returns 0 for shapes the pass does not take; dab_fconv_maxpool_pays (dabnn_hip_tuning.h) returns 1 when
  * the problem is also large enough on the current device for the pass to beat dab_fconv_affine_relu + dab_max_pool_sign.
  */
 DAB_API int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,
@@ -286,8 +259,6 @@ DAB_API int dab_fconv_maxpool(const float *x, int n, int h, int w, int c, const 
                               uint64_t *pooled_packed, float *carry, dab_stream_t stream);
 DAB_API int64_t dab_fconv_maxpool_carry_floats(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w,
                                                int stride_h, int stride_w, int dil_h, int dil_w, int cout);
-DAB_API int dab_fconv_maxpool_pays(int n, int h, int w, int c, int kh, int kw, int pad_h, int pad_w, int stride_h,
-                                   int stride_w, int dil_h, int dil_w, int cout);
 
 /* affine_inplace (dabnn/layers/Affine.cpp:10-23): x[..., ch] = a[ch]*x[..., ch] + b[ch]. */
 DAB_API int dab_affine_inplace(float *x, int64_t n_pix, int c, const float *a, const float *b, dab_stream_t stream);

@@ -10,9 +10,18 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "dabnn_hip.h")).read()
+def declared_symbols(headers=("dabnn_hip.h", "dabnn_hip_tuning.h")):
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in headers)
     return sorted(set(re.findall(r"^DAB_API [^;(]*?\b(dab_\w+)\(", text, flags=re.M)))
+
+
+def test_dispatch_probes_live_in_the_tuning_header():
+    """dabnn_hip.h is the reference's surface plus the documented extensions; the probes that only say which kernel
+    would run are declared in dabnn_hip_tuning.h."""
+    probes = declared_symbols(("dabnn_hip_tuning.h",))
+    assert probes == sorted(["dab_bconv3x3_build", "dab_bconv3x3_splits_depth", "dab_bconv3x3_fused_shares_tiles",
+                             "dab_global_ave_pool_fconv1x1_takes", "dab_fconv_maxpool_pays"])
+    assert not set(probes) & set(declared_symbols(("dabnn_hip.h",)))
 
 
 def test_header_declares_the_expected_entry_points():

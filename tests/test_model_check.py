@@ -161,3 +161,64 @@ def test_split_and_shuffle_want_bit_blobs(net):
     with pytest.raises(RuntimeError, match="Split only supports bit mat"):
         net.check_model(df.write_model([{"type": "Split", "name": "sp", "input": "data", "outputs": ["l", "r"]}], [],
                                        [("data", [1, 4, 4, 128])]))
+
+
+def test_a_layer_output_must_be_a_new_name(net):
+    """A layer that makes a blob (convolution, pool, concat, split) may not name it like a blob that exists: the net
+    would keep the existing blob, of another size, and the layer's kernel would write past it.  Checked on the host
+    only; such a model never reaches a device."""
+    layers, inits, inputs = small()
+    net.check_model(df.write_model(layers, inits, inputs))
+    convs = [i for i, l in enumerate(layers) if l["type"] in ("FpConv2D", "BinConv2D")]
+    binconvs = [i for i, l in enumerate(layers) if l["type"] == "BinConv2D"]
+    assert convs and binconvs
+
+    def renamed(index, new_name):
+        """layers with the output of layer `index` renamed, its readers following the new name."""
+        old = layers[index]["output"]
+        out = []
+        for i, l in enumerate(layers):
+            l = dict(l)
+            if i == index:
+                l["output"] = new_name
+            elif i > index:
+                for key in ("input", "input1", "input2"):
+                    if l.get(key) == old:
+                        l[key] = new_name
+            out.append(l)
+        return out
+
+    # a convolution's output named like the net's input
+    with pytest.raises(RuntimeError, match="already exists"):
+        net.check_model(df.write_model(renamed(convs[0], inputs[0][0]), inits, inputs))
+    # a BinConv's output named like an initializer (its own weight)
+    bc = binconvs[0]
+    with pytest.raises(RuntimeError, match="already exists"):
+        net.check_model(df.write_model(renamed(bc, layers[bc]["weight"]), inits, inputs))
+    # two BinConvs with the same output name would share the scratch blobs binaized_for_<out>_cal / col_for_<out>_cal
+    if len(binconvs) > 1:
+        with pytest.raises(RuntimeError, match="already exists"):
+            net.check_model(df.write_model(renamed(binconvs[1], layers[bc]["output"]), inits, inputs))
+    # an in-place layer re-pointing the input's name at another blob
+    inplace = [i for i, l in enumerate(layers) if l["type"] in ("Affine", "Relu", "Add")]
+    with pytest.raises(RuntimeError, match="already exists"):
+        net.check_model(df.write_model(renamed(inplace[-1], inputs[0][0]), inits, inputs))
+    # a later output named like a BinConv's scratch blob
+    pool = {"type": "MaxPool", "name": "late", "input": inputs[0][0], "output": "col_for_%s_cal" % layers[bc]["output"],
+            "kernel_shape": [2, 2], "pads": [0] * 4, "strides": [2, 2]}
+    with pytest.raises(RuntimeError, match="already exists"):
+        net.check_model(df.write_model(layers + [pool], inits, inputs))
+
+
+def test_window_extents_are_bounded(net):
+    """Kernel extents and output sizes that would overflow the int fields of the runtime are refused on the host."""
+    with pytest.raises(RuntimeError, match="too large"):
+        net.check_model(df.write_model([{"type": "MaxPool", "name": "p", "input": "data", "output": "o",
+                                         "kernel_shape": [1 << 16, 1], "pads": [32767, 0, 32767, 0], "strides": [1, 1]}], [],
+                                       [("data", [1, 12, 12, 64])]))
+    w = np.zeros((1 << 10, 1, 1, 4), np.float32)
+    conv = {"type": "FpConv2D", "name": "c", "input": "data", "weight": "w", "output": "o", "pads": [0] * 4,
+            "strides": [1, 1], "dilations": [1, 1]}
+    with pytest.raises(RuntimeError, match="too large"):
+        net.check_model(df.write_model([conv], [{"name": "w", "shape": list(w.shape), "data": w, "align_hwc_to_128": False}],
+                                       [("data", [1, 2048, 2048, 4])]))
