@@ -34,6 +34,10 @@ BATCH = 64
 # next to the algorithmic bytes (packed input + weights + fp32 output).
 TRAFFIC_BYTES_PER_LAUNCH = 26.52e6
 ALGORITHMIC_BYTES_PER_LAUNCH = 21.10e6
+# where the constant comes from: it is not measured by this run (the counters need rocprofv3 around the process) and
+# goes stale when the kernel changes, so the profile and the kernel sources it was collected on are named with it
+TRAFFIC_SOURCE = ("profiles/bconv3x3_config3_b64.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
+                  "`bench.py --profile-mode`), collected on dabnn_amd/csrc/bconv3x3.hip + xnor_core.h as of commit ca6ae4a")
 
 
 def out_dim(size, pad, k, stride):
@@ -201,15 +205,26 @@ def main():
     while time.perf_counter() - t_warm < 0.04:
         step_graph.replay()
         torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    step_graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    # The timed region is one replay of the graph (exactly K steps) between two events and two synchronisations; it is
+    # repeated, and the median replay is the one reported (minimum and maximum beside it).
+    REPLAYS = 11
+    walls, evs = [], []
+    for _ in range(REPLAYS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        step_graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+        evs.append(e0.elapsed_time(e1) * 1e-3)
+    order = sorted(range(REPLAYS), key=lambda i: walls[i])
+    mid = order[REPLAYS // 2]
+    wall = walls[mid]
     ms_per_step = wall * 1e3 / args.steps
     value = step_binops * args.steps / wall
+    event_seconds = sorted(evs)[REPLAYS // 2]
 
     # per-shape kernel durations (the roofline figure is launch-level)
     per_shape = []
@@ -220,12 +235,25 @@ def main():
         per_shape.append({"shape": "%dx%d %d->%d s%d b%d" % (hw, hw, cin, cout, stride, BATCH), "us": round(d * 1e6, 2),
                           "Tbinop/s": round(ops / d / 1e12, 1), "frac": round(ops / d / peak_binops, 3)})
     # launch-level roofline figure: all 7*K launches of the timed region (events around the graph launch)
-    step_seconds = e0.elapsed_time(e1) * 1e-3 / args.steps
+    step_seconds = event_seconds / args.steps
     achieved = step_binops / step_seconds
+    # The contract's peak prices a xor/popcount pair at 8 cycles per wave64 and SIMD (two full-rate instructions).  A
+    # register-only loop of the pair (v_xor_b32 with an SGPR operand, v_bcnt_u32_b32, strictly alternating, 4-8 waves
+    # per SIMD) issues in 6.36 cycles on this chip, so the kernels can exceed the contract's peak at large batch; the
+    # fraction against that measured issue rate is reported beside the contract's.
+    MEASURED_PAIR_CYCLES = 6.36
+    peak_measured_issue = peak_binops * 8.0 / MEASURED_PAIR_CYCLES
 
     workloads = {"config3_b64_per_shape_back_to_back": per_shape,
                  "config3_b64_back_to_back_frac": round(step_binops / dur_sum / peak_binops, 4),
-                 "config3_b64_events_ms_per_step": round(e0.elapsed_time(e1) / args.steps, 4)}
+                 "config3_b64_events_ms_per_step": round(event_seconds * 1e3 / args.steps, 4),
+                 "config3_b64_timed_replays": {
+                     "replays": REPLAYS, "steps_per_replay": args.steps,
+                     "wall_ms_per_step": {"median": round(ms_per_step, 5), "min": round(min(walls) * 1e3 / args.steps, 5),
+                                          "max": round(max(walls) * 1e3 / args.steps, 5)},
+                     "events_ms_per_step": {"median": round(event_seconds * 1e3 / args.steps, 5),
+                                            "min": round(min(evs) * 1e3 / args.steps, 5),
+                                            "max": round(max(evs) * 1e3 / args.steps, 5)}}}
 
     # ------------------------------------------------------------ config 3 at batch 1 and config 1
     b1 = []
@@ -233,13 +261,15 @@ def main():
         x, w = rand_words(1, hw, hw, cin // 64), rand_words(cout, 9 * cin // 64)
         d = timed(lambda: dab.bconv_3x3(x, w, stride, 1), 50)
         b1.append({"shape": "%dx%d %d->%d s%d b1" % (hw, hw, cin, cout, stride), "us": round(d * 1e6, 2),
-                   "Gbinop/s": round(binops(1, hw, cin, cout, stride) / d / 1e9, 1)})
+                   "Gbinop/s": round(binops(1, hw, cin, cout, stride) / d / 1e9, 1),
+                   "frac": round(binops(1, hw, cin, cout, stride) / d / peak_binops, 4)})
     workloads["config3_b1_per_shape"] = b1
     xf = torch.randn((1, 56, 56, 64), generator=g).cuda()
     layer = dab.BinConv(rand_words(64, 9), 3, 3, 1, 1, 1, 1)
     d = timed(lambda: layer(xf), 50)
     workloads["config1_binconv_fp32_in_b1"] = {"us": round(d * 1e6, 2),
-                                               "Gbinop/s": round(binops(1, 56, 64, 64, 1) / d / 1e9, 1)}
+                                               "Gbinop/s": round(binops(1, 56, 64, 64, 1) / d / 1e9, 1),
+                                               "frac": round(binops(1, 56, 64, 64, 1) / d / peak_binops, 4)}
 
     # ------------------------------------------------------------ config 2: standalone bitpack and bgemm
     xp = torch.randn((1, 56, 56, 512), generator=g).cuda()
@@ -273,7 +303,7 @@ def main():
         d = timed(lambda: layer(xf), 20)
         ops = binops(BATCH, hw, cin, cout, stride)
         full.append({"shape": "%dx%d %d->%d s%d b%d" % (hw, hw, cin, cout, stride, BATCH), "us": round(d * 1e6, 2),
-                     "Tbinop/s": round(ops / d / 1e12, 1)})
+                     "Tbinop/s": round(ops / d / 1e12, 1), "frac": round(ops / d / peak_binops, 3)})
     workloads["binconv_layer_fp32_in_b64"] = full
 
     # ------------------------------------------------------------ configs 4 and 5: Bi-Real-18 through the C++ Net
@@ -401,8 +431,15 @@ def main():
                    "device": torch.cuda.get_device_name(0),
                    "cus": cus, "clock_mhz": khz / 1e3},
         "roofline": {"bound": "valu_popcount", "achieved": achieved / 1e12, "peak": peak_binops / 1e12,
-                     "unit": "Tbinop/s", "frac": achieved / peak_binops, "traffic": TRAFFIC_BYTES_PER_LAUNCH,
+                     "unit": "Tbinop/s", "frac": achieved / peak_binops,
+                     "frac_at_measured_issue": achieved / peak_measured_issue,
+                     "peak_at_measured_issue": peak_measured_issue / 1e12,
+                     "measured_issue_note": "a register-only loop of the pair (v_xor_b32 with an SGPR operand + "
+                     "v_bcnt_u32_b32, strictly alternating, 4-8 waves per SIMD) issues in %.2f cycles per wave64 and SIMD "
+                     "where the contract's peak assumes 8" % MEASURED_PAIR_CYCLES,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH,
                      "traffic_algorithmic": ALGORITHMIC_BYTES_PER_LAUNCH,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "bconv3x3_kernel", "note": "peak = CUs*64 lanes*clock*32 binop (one v_xor_b32 + one "
                      "v_bcnt_u32_b32 per 32 bits); achieved = binops of the seven launches of a step / their HIP-event time "
                      "in the timed region (all K steps are one HIP graph; average launch = 1/7 of a step); traffic = HBM "

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "xnor_core.h"
+#include "bconv3x3_rows.h"
 
 namespace dab {
 
@@ -28,6 +29,7 @@ struct BconvArgs {
     int items_per_wave, items_extra;  // split of the work items over the waves
     uint32_t x_bytes;
     int half;      // HALF kernels: which 512 of the 1024 input channels (0 or 1)
+    int gran;      // row-split kernel: channels per work item (4, or 8 when sign bits are written)
     FastDiv div_ow, div_oh, div_groups;
     // fused epilogue (MODE >= 1 kernels only): out = a*cnt + b (+ shortcut); MODE 2 also writes sign bits of out
     const float *epi_a;
@@ -239,6 +241,154 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
     flush(std::integral_constant<int, 8>{}, cg, cg % WU);
 }
 
+// The row-split form (bconv3x3_rows.h): a block of three waves, wave r counting kernel row r of every output channel
+// of the block's segment; partial counts meet in LDS.
+template <int CW, int MODE>
+__global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
+    typedef RowSplit<CW> RS;
+    constexpr int DWR = RS::row_dwords, VEC = RS::vec, PIECES = RS::pieces, GROUP = RS::group, SEG = RS::segment, ROW = RS::row;
+    constexpr int kFilterBytes = 9 * CW * 8;  // one output channel's weights
+    constexpr int kPixelBytes = CW * 8;
+    __shared__ __attribute__((aligned(16))) unsigned char plane[64 * ROW];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int r = __builtin_amdgcn_readfirstlane(tid >> 6);  // this wave's kernel row
+
+    int i0, i1;
+    item_range((int)blockIdx.x, p.items_per_wave, p.items_extra, i0, i1);  // the block's items of p.gran channels
+    if (i0 >= i1) return;
+    int tile = (int)p.div_groups.div((uint32_t)i0);  // n_groups = items per tile
+    int ch = (i0 - tile * p.n_groups) * p.gran;
+    int left = (i1 - i0) * p.gran;
+    const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(p.x, p.x_bytes);
+
+    {
+        // Every wave walks the filters with scalar loads.  When other kernels have run in between they are in no L2
+        // any more, and the first wave of an XCD to need a row would wait for memory in the middle of its pass.  So
+        // the launch first touches every 128-byte line of the filters once per XCD (blocks are dealt to the eight
+        // XCDs in turn: block b runs on XCD b % 8): wave j of an XCD asks for one dword of each of the lines
+        // 64*j .. 64*j+63, straight into a sink in LDS, with no register involved.  The loads are done before the
+        // wave's first activations are (vector loads complete in order).
+        __shared__ uint32_t sink[RS::threads];
+        const uint32_t filter_bytes = (uint32_t)(p.cout * kFilterBytes);
+        const uint32_t n_lines = (filter_bytes + 127u) >> 7;
+        const uint32_t first = (uint32_t)((blockIdx.x >> 3) * 3 + r) * 64u;
+        if (first < n_lines) {
+            const uint32_t line = first + lane < n_lines ? first + lane : n_lines - 1;
+            const uint32_t byte = line * 128u < filter_bytes - 4u ? line * 128u : filter_bytes - 4u;
+            __builtin_amdgcn_global_load_lds(
+                (const void __attribute__((address_space(1))) *)(reinterpret_cast<const unsigned char *>(p.w) + byte),
+                (void __attribute__((address_space(3))) *)(sink + r * 64), 4, 0, 0);
+        }
+    }
+    uint32_t a[DWR];
+    int loaded_tile = -1;
+    bool plane_ready = false;
+    while (left > 0) {
+        int seg = p.cout - ch < SEG ? p.cout - ch : SEG;
+        seg = seg < left ? seg : left;
+        const int cbase = ch;  // first channel of the segment
+        if (tile != loaded_tile) {
+            loaded_tile = tile;
+            int pix = tile * 64 + lane;
+            pix = pix < p.total ? pix : p.total - 1;
+            const uint32_t t = p.div_ow.div(pix);
+            const int ox = pix - t * p.OW;
+            const uint32_t nimg = p.div_oh.div(t);
+            const int oy = t - nimg * p.OH;
+            const int y = oy * p.stride - p.pad + r, x0 = ox * p.stride - p.pad;
+            const int base = ((nimg * p.H + y) * p.W + x0) * kPixelBytes;  // byte offset of tap (r, 0); may be negative
+            const bool row_ok = (unsigned)y < (unsigned)p.H;
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const bool ok = row_ok && (unsigned)(x0 + kw) < (unsigned)p.W;
+                // an offset beyond the descriptor's range reads as zero: the reference's padding word
+                const int off = ok ? base + kw * kPixelBytes : (int)0x80000000;
+#pragma unroll
+                for (int c = 0; c < CW / 2; ++c) {
+                    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, c * 16, 0);
+                    uint32_t *dst = a + kw * CW * 2 + 4 * c;
+                    dst[0] = v.x, dst[1] = v.y, dst[2] = v.z, dst[3] = v.w;
+                }
+            }
+        }
+
+        if (!plane_ready) {
+            // the plane starts at zero (every store pass leaves it so); cleared behind the first loads, not before them
+            plane_ready = true;
+            for (int i = tid; i < 64 * ROW / 16; i += RS::threads) reinterpret_cast<u32x4 *>(plane)[i] = u32x4{0u, 0u, 0u, 0u};
+            __syncthreads();
+        }
+
+        // the whole-segment store pass's shortcut values, asked for before the counting so that they arrive behind it
+        float4 sc_pre[3];
+        bool pre_ok = false;
+        if constexpr (MODE == kModeAffineAdd || MODE == kModeAffineAddSign) {
+            if (p.epi_shortcut != nullptr && seg == SEG && (tile + 1) * 64 <= p.total) {
+                pre_ok = true;
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    const int pr = (tid >> 3) + j * (RS::threads / 8);
+                    sc_pre[j] = pr < 64 ? *reinterpret_cast<const float4 *>(p.epi_shortcut + ((size_t)tile * 64 + pr) * p.cout + cbase + (tid & 7) * 4)
+                                        : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+
+        {
+            // this wave's weights: row r of the segment's channels, GROUP channels per pass.  The scalar-load batches
+            // form one sequence (channel by channel, PIECES per channel) and batch j lives in wv[j & 1]: the one a body
+            // consumes was asked for by the body before it, also across passes (a pass is an even number of batches).
+            const unsigned char *wseg = reinterpret_cast<const unsigned char *>(p.w) + (size_t)cbase * kFilterBytes + r * (DWR * 4);
+            uint32_t *my = reinterpret_cast<uint32_t *>(plane + lane * ROW);
+            WVec<VEC> wv[2];
+            static_assert((GROUP * PIECES) % 2 == 0, "a pass starts with wv[0]");
+            const int groups = seg / GROUP;
+            uint32_t goff = 0;  // byte offset of the pass's first channel
+            wv[0].template load_off<0>(wseg, goff);
+            wv[0].wait();
+#pragma unroll 1
+            for (int g = 0; g < groups; ++g) {
+                uint32_t acc[GROUP];
+                const bool more = g + 1 < groups;
+                // (Wave priorities by remaining work, which help the unit kernel at three and four waves per SIMD, cost
+                // 0.3 us here: 16.8 against 16.4 us for 7 x 7 x 512 -> 512 at batch 64.)
+                static_for<GROUP * PIECES>([&](auto j_) {
+                    constexpr int j = j_, c = j / PIECES, piece = j % PIECES;
+                    constexpr int jn = j + 1, cn = jn / PIECES, pn = jn % PIECES;
+                    if constexpr (jn < GROUP * PIECES) {
+                        wv[jn & 1].template load_off<cn * kFilterBytes + pn * VEC * 4>(wseg, goff);
+                    } else {
+                        if (more) wv[0].template load_off<GROUP * kFilterBytes>(wseg, goff);
+                    }
+                    rows_count<VEC, piece == 0>(acc[c], wv[j & 1], a + piece * VEC);
+                    wv[jn & 1].wait();
+                });
+#pragma unroll
+                for (int c = 0; c < GROUP; ++c) atomicAdd(my + g * GROUP + c, acc[c]);
+                goff += GROUP * kFilterBytes;
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing of this wave is on its way into LDS any more
+        __syncthreads();
+        if constexpr (MODE == kModeAffineAddSign) {
+            EpiAffineAddSign epi;
+            epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+            epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+        } else if constexpr (MODE == kModeAffineAdd) {
+            EpiAffineAdd epi;
+            epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+        } else {
+            EpiStore epi;
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+        }
+        left -= seg, ch += seg;
+        if (ch == p.cout) ch = 0, ++tile;
+        if (left > 0) __syncthreads();  // the plane is zero again
+    }
+}
+
 // A few tiles only (small batches): the kernel above would leave most SIMDs without a
 // wave, each of the few waves grinding through all 4 or 8 input words of 9 taps.  Here a block is one work item of 64
 // pixels x 8 output channels and its four waves split the depth: a channel's 18*CW weight dwords (9 taps x CW words,
@@ -398,6 +548,28 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
+// Blocks per CU of the row-split kernel: six (18 waves) measured best at batch 64 (7 x 7 x 512 -> 512: 16.4 us with 6 to
+// 10, 17.2 with 4; 14 x 14 x 256 -> 512 at stride 2: 9.9 us with 6, 10.3-10.6 with 7 to 10).
+constexpr int kRowsBlocksPerCu = 6;
+
+template <int CW, int MODE>
+static int launch_rows(BconvArgs &a, long long tiles, hipStream_t stream) {
+    a.gran = MODE == kModeAffineAddSign ? 8 : 4;
+    a.n_groups = a.cout / a.gran;
+    const long long items = tiles * a.n_groups;
+    if (items >= (1ll << 31) / a.gran) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
+    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_rows_kernel<CW, MODE>, RowSplit<CW>::threads);
+    const int per_cu = blocks_per_cu < kRowsBlocksPerCu ? blocks_per_cu : kRowsBlocksPerCu;
+    long long blocks = (long long)(simd_count() / 4) * per_cu;
+    if (blocks > items) blocks = items;
+    a.items_per_wave = (int)(items / blocks);
+    a.items_extra = (int)(items % blocks);
+    a.div_groups = FastDiv((uint32_t)a.n_groups);
+    hipLaunchKernelGGL((bconv3x3_rows_kernel<CW, MODE>), dim3((unsigned)blocks), dim3(RowSplit<CW>::threads), 0, stream, a);
+    DAB_LAUNCH_CHECK();
+    return DAB_OK;
+}
+
 // 56 x 56 x 64 -> 64 with Affine, Add and sign bits inside Bi-Real-18: batch 128 (24 tiles per CU) level with the unit
 // kernel, batch 64 behind it, batch 256 (49): 87-91 us a launch against 87-100, the net 1.619 against 1.631 ms
 constexpr int kTile64MinTilesPerCu = 32;
@@ -528,10 +700,24 @@ static int launch_tile64(BconvArgs &a, long long tiles, hipStream_t stream) {
 
 // Which kernel runs a problem of `tiles` 64-pixel tiles: 0 = the small-problem kernel (blocks split the depth),
 // 1 = the unit kernel at its wide residency, 2 = its second build: four waves per SIMD and whole-line stores for 64
-// and 128 input channels, units of twice the channels for 256 and 512.
-constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2;
-static int pick_build(long long tiles, int cin, int cout) {
+// and 128 input channels, units of twice the channels for 256 and 512; 3 = the row-split kernel (raw counts only).
+constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2, kBuildRows = 3;
+
+// The row-split kernel takes mid-sized problems whose activation fetch is what the unit kernel waits for: 512 input
+// channels, and 256 at stride 2 (whose taps lie on twice as many cache lines), from the size where the small-problem
+// kernel ends up to 36 channel-tiles per SIMD (7 x 7 x 512 -> 512: 16.4 against 17.3 us at batch 64, 28.3 against
+// 28.6 at batch 128, 51.8 against 46.8 at batch 256; 14 x 14 x 256 -> 512 at stride 2: 6.8 against 7.9 us at batch
+// 32, 9.9 against 10.6 at batch 64, 16.1 against 16.0 at batch 128; 14 x 14 x 256 -> 256 at stride 1 is behind at
+// every batch).
+static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode) {
+    if (mode != kModeCounts || cout % 8 != 0) return false;
+    if (!(cin == 512 || (cin == 256 && stride >= 2))) return false;
+    return tiles * cout <= 36ll * simd_count();
+}
+
+static int pick_build(long long tiles, int cin, int cout, int stride = 1, int mode = kModeCounts) {
     if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
+    if (takes_rows(tiles, cin, cout, stride, mode)) return kBuildRows;
     if (cin <= 128) {
         // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (cout / 8);
@@ -549,8 +735,11 @@ static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     if constexpr (CW == 1 && (MODE == kModeAffineAdd || MODE == kModeAffineAddSign)) {
         if (takes_tile64(tiles, 64, a.cout, MODE)) return launch_tile64<MODE>(a, tiles, stream);
     }
-    const int build = pick_build(tiles, CW * 64, a.cout);
+    const int build = pick_build(tiles, CW * 64, a.cout, a.stride, MODE);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
+    if constexpr (CW >= 4 && MODE == kModeCounts) {
+        if (build == kBuildRows) return launch_rows<CW, MODE>(a, tiles, stream);
+    }
     if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
     return launch_variant<CW, MODE, false>(a, tiles, stream);
 }
@@ -661,5 +850,12 @@ extern "C" int dab_bconv3x3_fused_shares_tiles(int64_t n_out_pixels, int cin, in
 
 extern "C" int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout) {
     if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return -1;
-    return dab::pick_build((n_out_pixels + 63) / 64, cin, cout);
+    // the builds of the entry points with an epilogue; dab_bconv3x3_counts_build answers for dab_bconv3x3 itself
+    return dab::pick_build((n_out_pixels + 63) / 64, cin, cout, 1, dab::kModeAffineAdd);
 }
+
+extern "C" int dab_bconv3x3_counts_build(int64_t n_out_pixels, int cin, int cout, int stride) {
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || stride <= 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return -1;
+    return dab::pick_build((n_out_pixels + 63) / 64, cin, cout, stride, dab::kModeCounts);
+}
+

@@ -23,7 +23,7 @@ extern "C" {
 DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
 
 /*
- * Which of the three builds of the direct kernel dab_bconv3x3* runs for a problem of
+ * Which of the three builds of the direct kernel dab_bconv3x3_affine_add(_sign) runs for a problem of
  * n_out_pixels = N*OH*OW on the current device: 0 = the small-problem kernel (a block splits the depth over its
  * waves), 1 = the unit kernel's build for mid-sized problems, 2 = its build for large ones (four waves per SIMD and
  * whole-line stores for 64 and 128 input channels, units of twice the channels for 256 and 512; taken when a wave
@@ -31,6 +31,14 @@ DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
  * build it means to cover.
  */
 DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
+
+/*
+ * The same for dab_bconv3x3 itself (raw counts), which has a fourth build for mid-sized problems with 512 input
+ * channels, or 256 at a stride of 2 or more: 3 = the row-split kernel, whose blocks are three waves that count one
+ * kernel row each and add their partial counts in LDS.  dab_bconv3x3_build answers for the entry points with an
+ * epilogue, which never take it.
+ */
+DAB_API int dab_bconv3x3_counts_build(int64_t n_out_pixels, int cin, int cout, int stride);
 
 /*
  * Whether dab_bconv3x3_affine_add(_sign) runs a problem of n_out_pixels = N*OH*OW on

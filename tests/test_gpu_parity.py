@@ -297,6 +297,38 @@ def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, str
     np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
 
 
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,pad", [
+    # the shapes the row-split kernel is there for: 7 x 7 x 512 and the stride-2 layer into it, at batch 64 and 40
+    (64, 7, 7, 512, 512, 1, 1), (64, 14, 14, 256, 512, 2, 1), (44, 7, 7, 512, 512, 1, 1),
+    # a pixel count that is no multiple of 64, channel counts that are no multiple of a 32-channel segment, ranges
+    # of work that cross tiles in the middle of a segment
+    (200, 9, 7, 512, 88, 1, 1), (900, 7, 7, 512, 24, 1, 1), (130, 13, 11, 256, 104, 2, 1), (360, 5, 9, 512, 200, 2, 1),
+    # no padding, and a stride of 3
+    (340, 9, 9, 512, 64, 1, 0), (300, 15, 15, 256, 72, 3, 1),
+])
+def test_row_split_kernel_counts(dab, n, h, w, cin, cout, stride, pad):
+    """dab_bconv3x3 through its row-split build (blocks of three waves, one kernel row each, partial counts added in
+    LDS), named by the library so that the case cannot drift to another kernel: the whole batch against
+    baseline_bconv bit for bit."""
+    from dabnn_amd import capi
+    oh, ow = (h + 2 * pad - 3) // stride + 1, (w + 2 * pad - 3) // stride + 1
+    assert capi.lib.dab_bconv3x3_counts_build(n * oh * ow, cin, cout, stride) == 3
+    r = rng(31)
+    cw = cin // 64
+    x = r.integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    got = dab.bconv_3x3(dev_u(x), dev_u(wgt), stride, pad).cpu().numpy()
+    want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, pad, pad, stride, stride) for img in x])
+    np.testing.assert_array_equal(got, want)
+    # the entry points with an epilogue stay on the other builds and agree with it
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    fused = dab.bconv_3x3_affine_add(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), None, stride, pad)
+    sep = dev_f(want.copy())
+    dab.affine_inplace(sep, dev_f(a), dev_f(b))
+    assert torch.equal(fused, sep)
+
+
 @pytest.mark.parametrize("n,h,w,cin,cout,stride,build", [
     # the four-waves-per-SIMD build of the unit kernel (many units per wave): 128 input channels from 8 units per wave
     # on, 64 input channels from 4 -- the stage-2 and stage-1 blocks of Bi-Real-18 at batch 256

@@ -317,8 +317,8 @@ def test_bireal18_batch256_matches_cpu(mods, stem):
     """The benchmark's throughput configuration, both stems: at batch 256 other kernels run than at batch 2 or 64 (the
     four-waves-per-SIMD builds of the direct convolution with their epilogues, 64 x 256 tiles in the pooled shortcut
     convolutions, the one-pass stem without a carry launch, blocks with 512 input channels that leave the packing to
-    their successor).  Every layer group of the first and the last image against the CPU layers fed with the device's
-    own blobs, and every packed BinConv input against pack_mat of the blob it stands for."""
+    their successor).  Every layer group of nine images spread over the batch against the CPU layers fed with the
+    device's own blobs, and every packed BinConv input against pack_mat of the blob it stands for."""
     import torch
     df, models, net = mods
     from dabnn_amd import capi
@@ -340,9 +340,10 @@ def test_bireal18_batch256_matches_cpu(mods, stem):
     x = torch.randn((batch, 224, 224, 3), generator=gen).cuda()
     n.run(x)
     cached = CachedBlobs(n)
-    for i in (0, batch - 1):
-        assert check_every_segment(cached, layers, inits, i, gone) >= 19
-        assert check_packed_inputs(cached, layers, i) == 16
+    # images spread over the batch: a tile-indexing fault in the middle of a launch must not hide between the ends
+    for i in (0, 31, 63, 100, 127, 128, 191, 222, batch - 1):
+        assert check_every_segment(cached, layers, inits, i, gone) >= 19, i
+        assert check_packed_inputs(cached, layers, i) == 16, i
     first = cached.get_blob("logits").reshape(batch, -1).copy()
     cached.cache.clear()
     # a second and a third run (the third is the captured graph) give the same logits
