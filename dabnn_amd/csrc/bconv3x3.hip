@@ -538,7 +538,18 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     a.n_groups = a.cout / Q;
     const long long items = tiles * (a.n_groups / S);
     if (items >= (1ll << 31) / S) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
-    static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW, HALF>, 64 * kWavesPerBlock);
+    static const int resident = resident_blocks_per_cu(bconv3x3_kernel<CW, MODE, NARROW, HALF>, 64 * kWavesPerBlock);
+    int blocks_per_cu = resident;
+    if constexpr (CW == 1 && !NARROW) {
+        // 64 input channels: a unit is short (144 xor/popcount pairs) and a wave's fixed cost (arguments, pixel
+        // decode, nine taps, the store pass) weighs as much as a unit, so fewer, longer-lived waves are ahead as long
+        // as a wave's share still fits one 16-channel staging window (two units, one whole-window store pass): the
+        // fewest waves per SIMD that keep every share at two units or less.  56 x 56 x 64 -> 128 at stride 2, batch
+        // 64 (12 544 units): 9.5-9.8 us with 6 or 7 waves per SIMD against 10.3 with 8; 56 x 56 x 64 -> 64 at batch
+        // 24-36: 0.4-0.9 us less than with 8 (measured for every count from 4 to 8 at eight batch sizes each).
+        const long long per_simd = (items * S + 2ll * simd_count() - 1) / (2ll * simd_count());
+        if (items * S >= (long long)simd_count() * resident && per_simd < blocks_per_cu) blocks_per_cu = (int)per_simd;
+    }
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);
     a.items_extra = (int)(items % n_waves);
