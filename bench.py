@@ -89,7 +89,8 @@ def main():
     def timed(fn, reps, replays=5):
         """Average GPU duration of fn(): `reps` launches are captured into a HIP graph (so the Python/ctypes call
         overhead of ~10 us per launch does not throttle short kernels) and the graph is replayed between two
-        events on its launch stream."""
+        events on its launch stream, after untimed replays for 40 ms that let the shader clock settle -- the same
+        policy as the headline's timed region (an idle device runs its first milliseconds of load 5-10 % slower)."""
         fn()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -98,6 +99,10 @@ def main():
                 fn()
         graph.replay()
         torch.cuda.synchronize()
+        t_warm = time.perf_counter()
+        while time.perf_counter() - t_warm < 0.04:
+            graph.replay()
+            torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(replays):
