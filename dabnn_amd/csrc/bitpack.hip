@@ -4,35 +4,40 @@
 // x[64*i + j] > 0 (so +0, -0, NaN and negatives give 0).  On a 64-lane wave
 // that is exactly one v_cmp_gt_f32: the lane mask it produces IS the word.
 // A wave therefore reads 64 consecutive floats per instruction (256 coalesced
-// bytes), keeps the 64 masks of a 16 KiB chunk in lane i of a register pair
-// and writes them with one coalesced 512-byte store.  HBM-bound: 4 bytes read
-// and 1/16 byte written per element.  Every float is read once, so the loads
-// are non-temporal (411 MB: 69 instead of 78 us); the words are stored the
-// ordinary way, the next kernel reads them.
+// bytes), keeps the 16 masks of a 4 KiB chunk in lanes 0-15 of a register pair
+// and writes them with one 128-byte store.  HBM-bound: 4 bytes read and 1/16
+// byte written per element.  Every float is read once, so the loads are
+// non-temporal (411 MB: 69 instead of 78 us); the words are stored the ordinary
+// way, the next kernel reads them.  Chunks of 16 words, not 64: four times as
+// many waves in flight for the tensors of a single layer (25.7 MB: 3.8 instead
+// of 5.2 us, 6.6 MB: 2.2 instead of 3.0 us; 411 MB: 67 against 68 us; 8 words:
+// 64-byte stores, slower again from 13 MB up).
 #include "common.h"
 
 namespace dab {
 
 constexpr int kPackWavesPerBlock = 4;
 
+constexpr int kPackWords = 16;  // words per chunk of a wave
+
 __global__ __launch_bounds__(64 * kPackWavesPerBlock) void bitpack_nhwc_kernel(const float *__restrict__ x,
                                                                               uint64_t *__restrict__ out,
                                                                               long long n_words) {
     const int lane = threadIdx.x & 63;
     const long long wave = (long long)blockIdx.x * kPackWavesPerBlock + (threadIdx.x >> 6);
-    const long long n_chunks = (n_words + 63) / 64;
+    const long long n_chunks = (n_words + kPackWords - 1) / kPackWords;
     const long long stride = (long long)gridDim.x * kPackWavesPerBlock;
     for (long long chunk = wave; chunk < n_chunks; chunk += stride) {
-        const long long w0 = chunk * 64;
+        const long long w0 = chunk * kPackWords;
         const float *src = x + w0 * 64 + lane;
         uint64_t mine = 0;
-        if (w0 + 64 <= n_words) {
-#pragma unroll 16
-            for (int i = 0; i < 64; ++i) {
+        if (w0 + kPackWords <= n_words) {
+#pragma unroll
+            for (int i = 0; i < kPackWords; ++i) {
                 const uint64_t word = __ballot(__builtin_nontemporal_load(src + (long long)i * 64) > 0.0f);
                 mine = (lane == i) ? word : mine;
             }
-            out[w0 + lane] = mine;
+            if (lane < kPackWords) out[w0 + lane] = mine;
         } else {
             const int rem = (int)(n_words - w0);
             for (int i = 0; i < rem; ++i) {
@@ -144,7 +149,7 @@ extern "C" int dab_bitpack_nhwc(const float *x, uint64_t *out, int64_t n_pix, in
     DAB_REQUIRE(n_pix > 0 && c > 0, "dab_bitpack_nhwc: n_pix %lld c %d", (long long)n_pix, c);
     DAB_REQUIRE(c % 64 == 0, "dab_bitpack_nhwc: c %d is not a multiple of 64", c);
     const long long n_words = (long long)n_pix * (c / 64);
-    const long long chunks = (n_words + 63) / 64;
+    const long long chunks = (n_words + kPackWords - 1) / kPackWords;
     long long blocks = (chunks + kPackWavesPerBlock - 1) / kPackWavesPerBlock;
     const long long cap = (long long)simd_count() * 8;  // grid-stride beyond 8 waves per SIMD
     if (blocks > cap) blocks = cap;
