@@ -30,6 +30,7 @@ struct BconvArgs {
     uint32_t x_bytes;
     int half;      // HALF kernels: which 512 of the 1024 input channels (0 or 1)
     int gran;      // row-split kernel: channels per work item (4, or 8 when sign bits are written)
+    int through;   // raw counts through a 16-channel window: write-through stores instead of streaming ones
     FastDiv div_ow, div_oh, div_groups;
     // fused epilogue (MODE >= 1 kernels only): out = a*cnt + b (+ shortcut); MODE 2 also writes sign bits of out
     const float *epi_a;
@@ -152,8 +153,10 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
             stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
                                 (slot * Q + Q - 1) >> 2, epi);
         } else {
+            EpiStore epi;
+            epi.through = p.through;
             stage_flush<WCH, G>(stage, lane, p.out, p.cout, tile, p.total, (cg_now - slot) * Q, ch_lo >> 2,
-                                (slot * Q + Q - 1) >> 2, EpiStore());
+                                (slot * Q + Q - 1) >> 2, epi);
         }
     };
 
@@ -531,6 +534,11 @@ static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
+// Output sizes for which the 16-channel-window builds store write-through (stage_flush_window): measured on raw
+// counts of 56x56 64->64, 28x28 128->128, 56x56 64->128 and 28x28 128->256 (the last two at stride 2) at batches 16 to
+// 256: 0.2-1.0 us less per launch at 9.6-25.7 MB, 0.2-0.3 us more at 3-6 MB, level to 1.6x slower from 38 MB up.
+constexpr long long kThroughMinBytes = 9ll << 20, kThroughMaxBytes = 28ll << 20;
+
 template <int CW, int MODE, bool NARROW, bool HALF = false>
 static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     constexpr int Q = UnitChannels<CW, NARROW>::value;
@@ -549,6 +557,11 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
         // 24-36: 0.4-0.9 us less than with 8 (measured for every count from 4 to 8 at eight batch sizes each).
         const long long per_simd = (items * S + 2ll * simd_count() - 1) / (2ll * simd_count());
         if (items * S >= (long long)simd_count() * resident && per_simd < blocks_per_cu) blocks_per_cu = (int)per_simd;
+    }
+    if constexpr (Residency<CW, NARROW>::window == 16 && MODE == kModeCounts) {
+        // half-line runs of raw counts: written through when the output is a good part of the L2s and fits them
+        const long long out_bytes = 4ll * a.total * a.cout;
+        a.through = out_bytes >= kThroughMinBytes && out_bytes <= kThroughMaxBytes;
     }
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);
@@ -802,6 +815,7 @@ static int bconv3x3_impl(const char *fn, const uint64_t *x, int n, int h, int w,
     const long long tiles = (total + 63) / 64;
     hipStream_t s = as_stream(stream);
     a.half = 0;
+    a.through = 0;
     if (two_halves) {
         // the 512-channel unit kernel on words 0..7 of every pixel and tap, then on words 8..15 adding to the result
         // (the builds as for 512 channels; small problems take the unit kernel too)
