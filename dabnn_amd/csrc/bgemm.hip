@@ -50,7 +50,12 @@ __device__ __forceinline__ void add_to_c(float *__restrict__ c, int ldc, int row
         if (j >= j_first && row_ok) {
             float *d = c + (size_t)j * ldc + row;
             const float cnt = __uint_as_float(acc[q]) - kAccBias;
-            *d = overwrite ? cnt : *d + cnt;  // 0.f + cnt == cnt: the store alone is the fill + accumulate pair
+            // 0.f + cnt == cnt: the store alone is the fill + accumulate pair.  The accumulating form reads C when
+            // the count is done and wants it in the L2, where ordinary stores of an earlier launch leave it
+            if (overwrite)
+                store_through(d, cnt);
+            else
+                *d = *d + cnt;
         }
     }
 }
@@ -74,7 +79,7 @@ __device__ __forceinline__ void store_c(float *__restrict__ c, int ldc, int row,
         const int j = j0 + q;
         if (j >= j_first && row_ok) {
             const float cnt = __uint_as_float(acc[q]) - kAccBias;
-            c[(size_t)j * ldc + row] = old[q] + cnt;  // 0.f + cnt == cnt: the overwriting form never read C
+            store_through(c + (size_t)j * ldc + row, old[q] + cnt);  // 0.f + cnt == cnt: the overwriting form never read C
         }
     }
 }

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(64 * kPackWavesPerBlock) void bitpack_nhwc_kernel(c
                 const uint64_t word = __ballot(__builtin_nontemporal_load(src + (long long)i * 64) > 0.0f);
                 mine = (lane == i) ? word : mine;
             }
-            if (lane < kPackWords) out[w0 + lane] = mine;
+            if (lane < kPackWords) store_through(out + w0 + lane, mine);
         } else {
             const int rem = (int)(n_words - w0);
             for (int i = 0; i < rem; ++i) {

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(THREADS) void fused_binarize_im2col_tiled_kernel(co
         const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
         // a row inside the image is inside [y_lo, y_hi): the run's windows span exactly that range
         const bool ok = (int)tap < n_taps && y >= 0 && y < p.h && xx >= 0 && xx < p.w;
-        dst[g] = ok ? packed[((y - y_lo) * p.w + xx) * cw + k] : 0ull;
+        store_through(dst + g, ok ? packed[((y - y_lo) * p.w + xx) * cw + k] : 0ull);
     }
 }
 
