@@ -166,7 +166,8 @@ __device__ __forceinline__ void rows_flush(unsigned char *plane, int tid, float 
                             v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
                     else
                         r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
-                    *reinterpret_cast<float4 *>(out + off) = r;
+                    // the same kind of store as the whole-segment pass (a line finished by two kinds is written back twice)
+                    __builtin_nontemporal_store(f32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<f32x4 *>(out + off));
                     if constexpr (Epi::kEmit) nib = sign_nibble(r);
                 }
             }

@@ -42,11 +42,9 @@ __global__ __launch_bounds__(THREADS) void fused_binarize_im2col_tiled_kernel(co
     constexpr int WAVES = THREADS / 64;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wib = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Blocks are dealt to the eight XCDs in turn (block b runs on XCD b % 8) and every XCD has an L2 of its own:
-    // neighbouring runs of an image share their halo rows, so consecutive runs go to the same XCD and the second
-    // reader of a row finds it in that L2
-    int run_id = blockIdx.x;
-    if ((gridDim.x & 7) == 0) run_id = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    // neighbouring runs of an image share their halo rows: consecutive runs go to the same XCD, where the second
+    // reader of a row finds it in the L2 (64x28x28x128: 7.0 us against 8.2 with the runs dealt to the XCDs in turn)
+    const int run_id = (int)xcd_contiguous_block(blockIdx.x, gridDim.x);
     const int img = run_id / p.blocks_per_image, rb = run_id - img * p.blocks_per_image;
     const int cw = p.c >> 6;
     const int oy0 = rb * p.rows_per_block;

@@ -234,7 +234,7 @@ struct EpiStore {
     static constexpr bool kShortcut = false;  // the epilogue never reads a second tensor
     static constexpr bool kPolicy = true;     // the launch chooses how the stores go through the L2
     const float *shortcut = nullptr;
-    int through = 0;  // write-through stores (see stage_flush_window)
+    int through = 0;  // write-through stores: bit 0 whole 16-channel windows (stage_flush_window), bit 1 pieces of a window
     __device__ __forceinline__ void prepare(int) {}
     template <bool SC>
     __device__ __forceinline__ float4 apply(float4 v, float4) const {
@@ -362,9 +362,15 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
     constexpr int NP = Stage<WCH>::parts, ROW = Stage<WCH>::row;
     constexpr int GG = G < NP ? G : NP;
     const bool has_sc = Epi::kShortcut && epi.shortcut != nullptr;
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    // how the stores go through the L2 (EpiStore): bit 0 of the launch's choice is for whole 16-channel windows,
+    // bit 1 for the pieces of a window that a wave's range cuts off
+    bool through = false, parts_through = false;
+    if constexpr (Epi::kPolicy) {
+        through = WCH == 16 && (epi.through & 1) != 0;
+        parts_through = (epi.through & 2) != 0;
+    }
     if (np == NP && (tile + 1) * 64 <= total) {
-        bool through = false;
-        if constexpr (Epi::kPolicy && WCH == 16) through = epi.through != 0;
         if (has_sc)
             stage_flush_window<WCH, GG, Epi::kShortcut, false>(stage, lane, out, ld, tile, cbase, epi);
         else if (through)
@@ -389,7 +395,12 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
                         v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
                 else
                     r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
-                *reinterpret_cast<float4 *>(out + off) = r;
+                f32x4 *dst = reinterpret_cast<f32x4 *>(out + off);
+                const f32x4 rv = {r.x, r.y, r.z, r.w};
+                if (parts_through)
+                    store_through(dst, rv);
+                else
+                    *dst = rv;
                 if constexpr (Epi::kEmit) nib = sign_nibble(r);
             }
             if constexpr (Epi::kEmit) {
