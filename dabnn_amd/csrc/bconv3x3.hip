@@ -737,21 +737,25 @@ static int launch_tile64(BconvArgs &a, long long tiles, hipStream_t stream) {
 // and 128 input channels, units of twice the channels for 256 and 512; 3 = the row-split kernel (raw counts only).
 constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2, kBuildRows = 3;
 
-// The row-split kernel takes mid-sized problems whose activation fetch is what the unit kernel waits for: 512 input
-// channels, and 256 at stride 2 (whose taps lie on twice as many cache lines), from the size where the small-problem
-// kernel ends up to 36 channel-tiles per SIMD (7 x 7 x 512 -> 512: 16.4 against 17.3 us at batch 64, 28.3 against
-// 28.6 at batch 128, 51.8 against 46.8 at batch 256; 14 x 14 x 256 -> 512 at stride 2: 6.8 against 7.9 us at batch
-// 32, 9.9 against 10.6 at batch 64, 16.1 against 16.0 at batch 128; 14 x 14 x 256 -> 256 at stride 1 is behind at
-// every batch).
+// The row-split kernel takes the raw counts of deep inputs whose activation fetch is what the other kernels wait for,
+// from one tile up to 36 channel-tiles per SIMD with 512 input channels and with 256 at stride 2 (whose taps lie on
+// twice as many cache lines), and up to 16 with 256 channels at stride 1.  Against the small-problem kernel (batch 1
+// to 16) and the unit kernel: 7 x 7 x 512 -> 512: 3.9 against 4.6 us at batch 1, 6.8 against 7.6 at batch 16, 9.7
+// against 11.4 at batch 32, 15.7 against 17.0 at batch 64, 21.8 against 21.8 at batch 96, 30.0 against 27.7 at batch
+// 128; 14 x 14 x 256 -> 512 at stride 2: 3.1 against 3.8 us at batch 1, 4.7 against 6.1 at batch 16, 6.2 against 8.0 at
+// batch 32, 9.3 against 10.0 at batch 64, 12.7 against 12.3 at batch 96; 14 x 14 x 256 -> 256: 3.1 against 3.8 us at
+// batch 1, 6.0 against 7.0 at batch 16, 8.2 against 8.3 at batch 24, 11.4 against 9.9 at batch 40.  With an epilogue
+// the kernel is level or behind at most sizes (and with sign bits at every small one): raw counts only.
 static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode) {
     if (mode != kModeCounts || cout % 8 != 0) return false;
-    if (!(cin == 512 || (cin == 256 && stride >= 2))) return false;
-    return tiles * cout <= 36ll * simd_count();
+    if (cin == 512 || (cin == 256 && stride >= 2)) return tiles * cout <= 36ll * simd_count();
+    if (cin == 256) return tiles * cout <= 16ll * simd_count();
+    return false;
 }
 
 static int pick_build(long long tiles, int cin, int cout, int stride = 1, int mode = kModeCounts) {
-    if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
     if (takes_rows(tiles, cin, cout, stride, mode)) return kBuildRows;
+    if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
     if (cin <= 128) {
         // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (cout / 8);

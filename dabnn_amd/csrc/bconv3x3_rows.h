@@ -166,8 +166,12 @@ __device__ __forceinline__ void rows_flush(unsigned char *plane, int tid, float 
                             v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
                     else
                         r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
-                    // the same kind of store as the whole-segment pass (a line finished by two kinds is written back twice)
-                    __builtin_nontemporal_store(f32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<f32x4 *>(out + off));
+                    // Written through the L2 at device scope.  A block's share is 16 or 20 channels, so this is the
+                    // path nearly all of the kernel's output takes, in pieces of a line; as ordinary or streaming
+                    // stores the pieces wait in the L2 for the rest of their line, which another block writes at
+                    // another time.  14x14 256->512 at stride 2: 6.1 against 7.9 us at batch 32, 9.15 against 9.7 at
+                    // batch 64; 7x7 512->512 at batch 64: 15.7 against 16.6.
+                    store_through(reinterpret_cast<f32x4 *>(out + off), f32x4{r.x, r.y, r.z, r.w});
                     if constexpr (Epi::kEmit) nib = sign_nibble(r);
                 }
             }

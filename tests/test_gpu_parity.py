@@ -305,6 +305,10 @@ def test_bconv_affine_add_sign_packs_its_own_output(dab, n, h, w, cin, cout, str
     (200, 9, 7, 512, 88, 1, 1), (900, 7, 7, 512, 24, 1, 1), (130, 13, 11, 256, 104, 2, 1), (360, 5, 9, 512, 200, 2, 1),
     # no padding, and a stride of 3
     (340, 9, 9, 512, 64, 1, 0), (300, 15, 15, 256, 72, 3, 1),
+    # small batches, where it runs in place of the small-problem kernel: one image of the three deep stage shapes,
+    # a single tile that is not full, eight output channels, 256 input channels at stride 1 up to its bound
+    (1, 7, 7, 512, 512, 1, 1), (1, 14, 14, 256, 256, 1, 1), (1, 14, 14, 256, 512, 2, 1), (3, 7, 7, 512, 40, 1, 1),
+    (2, 5, 5, 256, 8, 1, 1), (16, 14, 14, 256, 256, 1, 1), (20, 14, 14, 256, 256, 1, 1),
 ])
 def test_row_split_kernel_counts(dab, n, h, w, cin, cout, stride, pad):
     """dab_bconv3x3 through its row-split build (blocks of three waves, one kernel row each, partial counts added in
