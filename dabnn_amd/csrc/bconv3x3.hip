@@ -539,8 +539,10 @@ static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
 // 256: 0.2-1.0 us less per launch at 9.6-25.7 MB, 0.2-0.3 us more at 3-6 MB, level to 1.6x slower from 38 MB up.
 // Pieces of a window (every build): 14x14 256->256 at batch 64 (12.8 MB) 13.8 us written through, 14.5 as streaming
 // and 15.1 as ordinary stores; 14x14 256->512 at stride 2 and batch 256 (25.7 MB) 23.9 / 26.4 / 26.6; from 51 MB up
-// ordinary stores are level or ahead (56x56 64->128 at stride 2, batch 256: 26.4 against 28.3 written through), and
-// below 6 MB (9 MB with 16-channel windows) they are 0.3-0.6 us ahead.
+// with 16-channel windows ordinary stores are ahead (56x56 64->128 at stride 2, batch 256: 26.4 against 28.3 written
+// through), with 32-channel windows the written-through pieces stay level or ahead (56x56 64->64 at batch 64, 51 MB:
+// 16.05 against 16.4; at batch 256, 205 MB: 52.5 against 52.3); below 6 MB (9 MB with 16-channel windows) ordinary
+// stores are 0.3-0.6 us ahead.
 constexpr long long kPartsThroughMinBytes = 6ll << 20;
 constexpr long long kThroughMinBytes = 9ll << 20, kThroughMaxBytes = 28ll << 20;
 
@@ -569,9 +571,11 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
         // half-line runs of raw counts: written through when the output is a good part of the L2s and fits them
         if (Residency<CW, NARROW>::window == 16 && out_bytes >= kThroughMinBytes && out_bytes <= kThroughMaxBytes) a.through |= 1;
         // the pieces of a window at the ends of a wave's range (most of the stores when a wave has fewer units than
-        // a window, as with 256 input channels at batch 64): written through while the output fits the L2s
-        const long long parts_min = Residency<CW, NARROW>::window == 16 ? kThroughMinBytes : kPartsThroughMinBytes;
-        if (out_bytes >= parts_min && out_bytes <= kThroughMaxBytes) a.through |= 2;
+        // a window, as with 256 input channels at batch 64): written through, with 16-channel windows while the
+        // output fits the L2s, with 32-channel windows at any size above the small ones
+        if (Residency<CW, NARROW>::window == 16 ? (out_bytes >= kThroughMinBytes && out_bytes <= kThroughMaxBytes)
+                                                : out_bytes >= kPartsThroughMinBytes)
+            a.through |= 2;
     }
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);
