@@ -249,6 +249,10 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
 template <int CW, int MODE>
 __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
     typedef RowSplit<CW> RS;
+    // Raw counts only.  The store pass is written for every epilogue, but the builds with one are not shipped: with
+    // Affine + Add they are level with the other kernels at most sizes, and the build that also writes sign bits
+    // disagreed with the CPU layers on mid-sized problems in a trial (cause not found), so it must not be dispatched.
+    static_assert(MODE == kModeCounts, "the row-split kernel is verified for raw counts only");
     constexpr int DWR = RS::row_dwords, VEC = RS::vec, PIECES = RS::pieces, GROUP = RS::group, SEG = RS::segment, ROW = RS::row;
     constexpr int kFilterBytes = 9 * CW * 8;  // one output channel's weights
     constexpr int kPixelBytes = CW * 8;
