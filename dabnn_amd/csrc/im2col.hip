@@ -28,6 +28,8 @@ struct Im2colArgs {
     long long n_words;
     FastDiv div_row_words, div_ow, div_oh, div_c, div_kw, div_cw;
     int rows_per_block, blocks_per_image;  // tiled kernel only
+    int packed_words;                      // tiled kernel: words of packed input rows a block holds in LDS
+    int step_wi, step_ox, step_oy;         // tiled kernel: what 512 words further on means for (index in row, ox, oy)
 };
 
 constexpr int kIm2colWavesPerBlock = 4;
@@ -82,24 +84,38 @@ __global__ __launch_bounds__(THREADS) void fused_binarize_im2col_tiled_kernel(co
         }
         if (lane < cnt) packed[j0 + lane] = mine;
     }
-    __syncthreads();
-    uint64_t *dst = p.col + ((size_t)img * p.oh + oy0) * p.ow * p.row_words;
-    const int n_taps = p.kh * p.kw;
-    const int n_out = (oy1 - oy0) * p.ow * p.row_words;
-    for (int g = tid; g < n_out; g += THREADS) {
-        const uint32_t pix = p.div_row_words.div((uint32_t)g);
-        const int wi = g - pix * p.row_words;
-        const uint32_t oyl = p.div_ow.div(pix);
-        const int ox = pix - oyl * p.ow;
+    // What a word of a col row gathers depends on its index in the row alone: tap (row and column offset of the
+    // window) and channel word, decoded once per block into a table behind the packed rows.  Entry: x = the tap's row
+    // offset (far outside every image for the zero padding word), y = column offset * 4096 + channel word.
+    int2 *word_tab = reinterpret_cast<int2 *>(packed + p.packed_words);
+    for (int wi = tid; wi < p.row_words; wi += THREADS) {
         const uint32_t tap = p.div_cw.div((uint32_t)wi);  // >= kh*kw for the zero padding word
         const int k = wi - tap * cw;
         const uint32_t a = p.div_kw.div(tap);
         const int b = tap - a * p.kw;
-        const int y = (oy0 + (int)oyl) * p.stride_h - p.pad_h + (int)a * p.dil_h;
-        const int xx = ox * p.stride_w - p.pad_w + b * p.dil_w;
+        word_tab[wi] = make_int2((int)tap < p.kh * p.kw ? (int)a * p.dil_h - p.pad_h : -(1 << 20), (b * p.dil_w - p.pad_w) * 4096 + k);
+    }
+    __syncthreads();
+    uint64_t *dst = p.col + ((size_t)img * p.oh + oy0) * p.ow * p.row_words;
+    const int n_out = (oy1 - oy0) * p.ow * p.row_words;
+    // word g = tid + i * THREADS of the run: pixel and index in the row advance by constants, no division in the loop
+    uint32_t pix0 = p.div_row_words.div((uint32_t)tid);
+    int wi = tid - (int)pix0 * p.row_words;
+    int oyl = (int)p.div_ow.div(pix0);
+    int ox = (int)pix0 - oyl * p.ow;
+    for (int g = tid; g < n_out; g += THREADS) {
+        const int2 e = word_tab[wi];
+        const int y = (oy0 + oyl) * p.stride_h + e.x;
+        const int xx = ox * p.stride_w + (e.y >> 12);
         // a row inside the image is inside [y_lo, y_hi): the run's windows span exactly that range
-        const bool ok = (int)tap < n_taps && y >= 0 && y < p.h && xx >= 0 && xx < p.w;
-        store_through(dst + g, ok ? packed[((y - y_lo) * p.w + xx) * cw + k] : 0ull);
+        const bool ok = y >= 0 && y < p.h && xx >= 0 && xx < p.w;
+        store_through(dst + g, ok ? packed[((y - y_lo) * p.w + xx) * cw + (e.y & 4095)] : 0ull);
+        wi += p.step_wi;
+        const int carry = wi >= p.row_words ? 1 : 0;
+        wi -= carry ? p.row_words : 0;
+        ox += p.step_ox + carry;
+        oyl += p.step_oy;
+        if (ox >= p.ow) ox -= p.ow, ++oyl;
     }
 }
 
@@ -228,7 +244,7 @@ extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, in
         // 14x14x256 and 7x7x512 with every candidate: the estimate picks the fastest or one within 3 % of it.
         const int cw = c / 64;
         auto in_rows = [&](int r) { return (long long)(r - 1) * stride_h + (long long)(kh - 1) * dil_h + 1; };
-        auto lds_bytes = [&](int r) { return in_rows(r) * w * cw * 8; };
+        auto lds_bytes = [&](int r) { return (in_rows(r) * w * cw + a.row_words) * 8; };  // packed rows + the word table
         const long long cus = simd_count() / 4;
         int r = 1;
         double best = 0.0;
@@ -241,6 +257,9 @@ extern "C" int dab_fused_binarize_im2col(const float *x, int n, int h, int w, in
         if (lds_bytes(r) <= 48 * 1024) {
             a.rows_per_block = r;
             a.blocks_per_image = (a.oh + r - 1) / r;
+            a.packed_words = (int)(in_rows(r) * w * cw);
+            const int step_pix = 512 / a.row_words;
+            a.step_wi = 512 % a.row_words, a.step_ox = step_pix % a.ow, a.step_oy = step_pix / a.ow;
             hipLaunchKernelGGL(fused_binarize_im2col_tiled_kernel<512>, dim3((unsigned)(n * a.blocks_per_image)), dim3(512),
                                (size_t)lds_bytes(r), as_stream(stream), a);
             DAB_LAUNCH_CHECK();
