@@ -30,7 +30,7 @@ struct BconvArgs {
     uint32_t x_bytes;
     int half;      // HALF kernels: which 512 of the 1024 input channels (0 or 1)
     int gran;      // row-split kernel: channels per work item (4, or 8 when sign bits are written)
-    int through;   // raw counts through a 16-channel window: write-through stores instead of streaming ones
+    int through;   // raw counts: written through the L2 instead of as streaming (windows) and ordinary (pieces) stores
     FastDiv div_ow, div_oh, div_groups;
     // fused epilogue (MODE >= 1 kernels only): out = a*cnt + b (+ shortcut); MODE 2 also writes sign bits of out
     const float *epi_a;
@@ -538,17 +538,16 @@ static int launch_ksplit(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
-// Output sizes for which the 16-channel-window builds store write-through (stage_flush_window): measured on raw
-// counts of 56x56 64->64, 28x28 128->128, 56x56 64->128 and 28x28 128->256 (the last two at stride 2) at batches 16 to
-// 256: 0.2-1.0 us less per launch at 9.6-25.7 MB, 0.2-0.3 us more at 3-6 MB, level to 1.6x slower from 38 MB up.
-// Pieces of a window (every build): 14x14 256->256 at batch 64 (12.8 MB) 13.8 us written through, 14.5 as streaming
-// and 15.1 as ordinary stores; 14x14 256->512 at stride 2 and batch 256 (25.7 MB) 23.9 / 26.4 / 26.6; from 51 MB up
-// with 16-channel windows ordinary stores are ahead (56x56 64->128 at stride 2, batch 256: 26.4 against 28.3 written
-// through), with 32-channel windows the written-through pieces stay level or ahead (56x56 64->64 at batch 64, 51 MB:
-// 16.05 against 16.4; at batch 256, 205 MB: 52.5 against 52.3); below 6 MB (9 MB with 16-channel windows) ordinary
-// stores are 0.3-0.6 us ahead.
-constexpr long long kPartsThroughMinBytes = 6ll << 20;
-constexpr long long kThroughMinBytes = 9ll << 20, kThroughMaxBytes = 28ll << 20;
+// Raw counts are written through the L2 (stage_flush, stage_flush_window) when the output is larger than this: 9 MB
+// for the builds with 16-channel windows, 6 MB for those with 32-channel windows; below it the whole windows are
+// streaming stores and the pieces ordinary ones (0.2-0.6 us less per launch at 1.6-6 MB).  All stores of a launch go
+// one way: a line that one wave finishes with one kind of store and another wave with another is written back twice,
+// and written-through windows beside ordinary pieces took up to 1.6x as long from 38 MB up.  Measured on the seven
+// stage shapes at batches 8 to 256 against streaming windows + ordinary pieces: 28x28 128->128 13.3 against 14.5 us at
+// batch 64, 24.2 against 26.5 at batch 128; 56x56 64->64 14.6 against 16.2 at batch 64; 14x14 256->256 13.8 against
+// 15.1; 56x56 64->128 at stride 2 8.7 against 9.6; 28x28 128->256 at stride 2 24.5 against 27.2 at batch 256; the
+// seven-shape step 84.0 against 93.1 us at batch 64 and 261 against 267 at batch 256.
+constexpr long long kThroughMinBytes16 = 9ll << 20, kThroughMinBytes32 = 6ll << 20;
 
 template <int CW, int MODE, bool NARROW, bool HALF = false>
 static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
@@ -572,14 +571,7 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     if constexpr (MODE == kModeCounts) {
         const long long out_bytes = 4ll * a.total * a.cout;
         a.through = 0;
-        // half-line runs of raw counts: written through when the output is a good part of the L2s and fits them
-        if (Residency<CW, NARROW>::window == 16 && out_bytes >= kThroughMinBytes && out_bytes <= kThroughMaxBytes) a.through |= 1;
-        // the pieces of a window at the ends of a wave's range (most of the stores when a wave has fewer units than
-        // a window, as with 256 input channels at batch 64): written through, with 16-channel windows while the
-        // output fits the L2s, with 32-channel windows at any size above the small ones
-        if (Residency<CW, NARROW>::window == 16 ? (out_bytes >= kThroughMinBytes && out_bytes <= kThroughMaxBytes)
-                                                : out_bytes >= kPartsThroughMinBytes)
-            a.through |= 2;
+        if (out_bytes >= (Residency<CW, NARROW>::window == 16 ? kThroughMinBytes16 : kThroughMinBytes32)) a.through = 1;
     }
     const int n_waves = pick_wave_count((int)items, blocks_per_cu, kWavesPerBlock, S);
     a.items_per_wave = (int)(items / n_waves);

@@ -234,7 +234,7 @@ struct EpiStore {
     static constexpr bool kShortcut = false;  // the epilogue never reads a second tensor
     static constexpr bool kPolicy = true;     // the launch chooses how the stores go through the L2
     const float *shortcut = nullptr;
-    int through = 0;  // write-through stores: bit 0 whole 16-channel windows (stage_flush_window), bit 1 pieces of a window
+    int through = 0;  // write-through stores (see stage_flush_window)
     __device__ __forceinline__ void prepare(int) {}
     template <bool SC>
     __device__ __forceinline__ float4 apply(float4 v, float4) const {
@@ -290,14 +290,13 @@ struct EpiAffineAddSign : EpiAffineAdd {
 // flush waits for memory NP/G times and not once per store (the loads of one store cannot move above the previous
 // store by themselves: the compiler has to assume the two tensors overlap).
 //
-// THROUGH: the stores are write-through at device scope (sc1) instead of streaming (nt).  A 16-channel window
-// writes 64-byte runs, half a line; as streaming stores the halves wait in the L2 for each other, part of them is
-// written back twice (the write counter reads 9-17 % above the output) and what is still there when the kernel
-// ends is written back before the next kernel starts.  Written through, every run leaves the L2 once, as it
-// arrives: the counter reads the output size, and launches whose output is a good part of the L2s but fits them
-// (9-28 MB against 8 x 4 MB) end 0.3-1.0 us earlier (batch 64, 28x28 128->128: 13.6 against 14.5 us; 56x56 64->128
-// at stride 2: 8.9 against 9.6).  Larger outputs take up to 1.6x as long that way, smaller ones 0.2-0.3 us more,
-// so the launcher asks for it inside that window only.
+// THROUGH: the stores are write-through at device scope (sc1) instead of streaming (nt).  A kernel's end waits until
+// every dirty line it left in the L2s is written back, and the halves of a line that two store instructions fill
+// (64-byte runs of a 16-channel window) or two waves (the pieces at the ends of their ranges) wait there for each
+// other; part of them is written back twice (the write counter read 9-17 % above the output).  Written through,
+// every piece leaves the L2 once, as it arrives: the counter reads the output size, a launch ends 0.3-1.6 us earlier
+// at batch 64 and the next one starts on an L2 with nothing left to write.  Small outputs stay in the L2s either
+// way and are 0.2-0.6 us faster with the streaming stores, so the launcher asks for this above a size.
 template <int WCH, int G, bool SC, bool THROUGH, class Epi>
 __device__ __forceinline__ void stage_flush_window(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
                                                    int tile, int cbase, Epi &epi) {
@@ -363,18 +362,15 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
     constexpr int GG = G < NP ? G : NP;
     const bool has_sc = Epi::kShortcut && epi.shortcut != nullptr;
     typedef float f32x4 __attribute__((ext_vector_type(4)));
-    // how the stores go through the L2 (EpiStore): bit 0 of the launch's choice is for whole 16-channel windows,
-    // bit 1 for the pieces of a window that a wave's range cuts off
-    bool through = false, parts_through = false;
-    if constexpr (Epi::kPolicy) {
-        through = WCH == 16 && (epi.through & 1) != 0;
-        parts_through = (epi.through & 2) != 0;
-    }
+    // how the stores go through the L2 is the launch's choice (EpiStore), one way for all of them
+    bool through = false;
+    if constexpr (Epi::kPolicy) through = epi.through != 0;
+    const bool parts_through = through;
     if (np == NP && (tile + 1) * 64 <= total) {
         if (has_sc)
             stage_flush_window<WCH, GG, Epi::kShortcut, false>(stage, lane, out, ld, tile, cbase, epi);
         else if (through)
-            stage_flush_window<WCH, GG, false, Epi::kPolicy && WCH == 16>(stage, lane, out, ld, tile, cbase, epi);
+            stage_flush_window<WCH, GG, false, Epi::kPolicy>(stage, lane, out, ld, tile, cbase, epi);
         else
             stage_flush_window<WCH, GG, false, false>(stage, lane, out, ld, tile, cbase, epi);
     } else {
