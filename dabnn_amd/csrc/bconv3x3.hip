@@ -738,17 +738,17 @@ static int launch_tile64(BconvArgs &a, long long tiles, hipStream_t stream) {
 constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2, kBuildRows = 3;
 
 // The row-split kernel takes the raw counts of deep inputs whose activation fetch is what the other kernels wait for,
-// from one tile up to 36 channel-tiles per SIMD with 512 input channels and with 256 at stride 2 (whose taps lie on
+// from one tile up to 28 channel-tiles per SIMD with 512 input channels and with 256 at stride 2 (whose taps lie on
 // twice as many cache lines), and up to 16 with 256 channels at stride 1.  Against the small-problem kernel (batch 1
 // to 16) and the unit kernel: 7 x 7 x 512 -> 512: 3.9 against 4.6 us at batch 1, 6.8 against 7.6 at batch 16, 9.7
-// against 11.4 at batch 32, 15.7 against 17.0 at batch 64, 21.8 against 21.8 at batch 96, 30.0 against 27.7 at batch
+// against 11.4 at batch 32, 15.7 against 17.0 at batch 64, 19.2 against 18.6 at batch 80, 30.0 against 27.7 at batch
 // 128; 14 x 14 x 256 -> 512 at stride 2: 3.1 against 3.8 us at batch 1, 4.7 against 6.1 at batch 16, 6.2 against 8.0 at
-// batch 32, 9.3 against 10.0 at batch 64, 12.7 against 12.3 at batch 96; 14 x 14 x 256 -> 256: 3.1 against 3.8 us at
+// batch 32, 9.3 against 10.1 at batch 64, 11.4 against 11.1 at batch 80; 14 x 14 x 256 -> 256: 3.1 against 3.8 us at
 // batch 1, 6.0 against 7.0 at batch 16, 8.2 against 8.3 at batch 24, 11.4 against 9.9 at batch 40.  With an epilogue
 // the kernel is level or behind at most sizes (and with sign bits at every small one): raw counts only.
 static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode) {
     if (mode != kModeCounts || cout % 8 != 0) return false;
-    if (cin == 512 || (cin == 256 && stride >= 2)) return tiles * cout <= 36ll * simd_count();
+    if (cin == 512 || (cin == 256 && stride >= 2)) return tiles * cout <= 28ll * simd_count();
     if (cin == 256) return tiles * cout <= 16ll * simd_count();
     return false;
 }
