@@ -252,7 +252,9 @@ __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
     // Raw counts only.  The store pass is written for every epilogue, but the builds with one are not shipped: with
     // Affine + Add they are level with the other kernels at most sizes, and the build that also writes sign bits
     // disagreed with the CPU layers on mid-sized problems in a trial (cause not found), so it must not be dispatched.
+#ifndef DAB_ROWS_DEBUG
     static_assert(MODE == kModeCounts, "the row-split kernel is verified for raw counts only");
+#endif
     constexpr int DWR = RS::row_dwords, VEC = RS::vec, PIECES = RS::pieces, GROUP = RS::group, SEG = RS::segment, ROW = RS::row;
     constexpr int kFilterBytes = 9 * CW * 8;  // one output channel's weights
     constexpr int kPixelBytes = CW * 8;
@@ -754,6 +756,9 @@ static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode)
 }
 
 static int pick_build(long long tiles, int cin, int cout, int stride = 1, int mode = kModeCounts) {
+#ifdef DAB_ROWS_DEBUG
+    if (cin >= 256 && cout % 8 == 0 && (mode != kModeAffineAddSign || cout % 64 == 0)) return kBuildRows;
+#endif
     if (takes_rows(tiles, cin, cout, stride, mode)) return kBuildRows;
     if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
     if (cin <= 128) {
@@ -775,7 +780,11 @@ static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     }
     const int build = pick_build(tiles, CW * 64, a.cout, a.stride, MODE);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
+#ifdef DAB_ROWS_DEBUG
+    if constexpr (CW >= 4) {
+#else
     if constexpr (CW >= 4 && MODE == kModeCounts) {
+#endif
         if (build == kBuildRows) return launch_rows<CW, MODE>(a, tiles, stream);
     }
     if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);

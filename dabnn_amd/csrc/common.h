@@ -111,7 +111,10 @@ __device__ __forceinline__ void store_through(T *p, const U &value) {
     else if constexpr (sizeof(T) == 8)
         asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
     else
-        asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+        // A store of more than 8 bytes still reads its data registers for two cycles after it has issued, and a
+        // vector instruction that overwrites them in that time changes what is stored.  The compiler keeps that
+        // distance for the stores it emits itself; it cannot see into this statement, so the statement keeps it.
+        asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
 }
 
 // ---------------------------------------------------------------- sign bits of results

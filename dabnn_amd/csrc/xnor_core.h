@@ -327,7 +327,7 @@ __device__ __forceinline__ void stage_flush_window(const unsigned char *stage, i
             const f32x4 rv = {r.x, r.y, r.z, r.w};
             f32x4 *dst = reinterpret_cast<f32x4 *>(out + off0 + (size_t)i * PPI * ld);
             if constexpr (THROUGH)
-                asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(dst), "v"(rv) : "memory");
+                store_through(dst, rv);
             else
                 // streaming store: the output is not read again by this kernel, and lines that leave the L2 early
                 // do not have to be written back when the kernel ends
