@@ -249,12 +249,11 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
 template <int CW, int MODE>
 __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
     typedef RowSplit<CW> RS;
-    // Raw counts only.  The store pass is written for every epilogue, but the builds with one are not shipped: with
-    // Affine + Add they are level with the other kernels at most sizes, and the build that also writes sign bits
-    // disagreed with the CPU layers on mid-sized problems in a trial (cause not found), so it must not be dispatched.
-#ifndef DAB_ROWS_DEBUG
-    static_assert(MODE == kModeCounts, "the row-split kernel is verified for raw counts only");
-#endif
+    // Raw counts only in the dispatch.  The store pass is written for every epilogue and the builds with one agree
+    // with the CPU layers on every case of the parity tests when they are forced onto them; against the other kernels
+    // they are behind at batch 1-4 with sign bits and at batch 256, and 5-30 % ahead between batch 8 and 64, which
+    // the dispatch (and the net's choice of who writes the sign bits) does not use yet.
+    static_assert(MODE == kModeCounts, "the row-split kernel is dispatched for raw counts only");
     constexpr int DWR = RS::row_dwords, VEC = RS::vec, PIECES = RS::pieces, GROUP = RS::group, SEG = RS::segment, ROW = RS::row;
     constexpr int kFilterBytes = 9 * CW * 8;  // one output channel's weights
     constexpr int kPixelBytes = CW * 8;
@@ -756,9 +755,6 @@ static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode)
 }
 
 static int pick_build(long long tiles, int cin, int cout, int stride = 1, int mode = kModeCounts) {
-#ifdef DAB_ROWS_DEBUG
-    if (cin >= 256 && cout % 8 == 0 && (mode != kModeAffineAddSign || cout % 64 == 0)) return kBuildRows;
-#endif
     if (takes_rows(tiles, cin, cout, stride, mode)) return kBuildRows;
     if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
     if (cin <= 128) {
@@ -780,11 +776,7 @@ static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     }
     const int build = pick_build(tiles, CW * 64, a.cout, a.stride, MODE);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
-#ifdef DAB_ROWS_DEBUG
-    if constexpr (CW >= 4) {
-#else
     if constexpr (CW >= 4 && MODE == kModeCounts) {
-#endif
         if (build == kBuildRows) return launch_rows<CW, MODE>(a, tiles, stream);
     }
     if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);

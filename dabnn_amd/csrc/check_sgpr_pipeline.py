@@ -8,6 +8,11 @@ lane, s_mov_b32 to another SGPR), it would move garbage and the kernel would cou
 script reads the device assembly the compiler produced (hipcc --save-temps) and fails the build when any instruction
 reads an SGPR of a scalar load issued from inline asm before the next `s_waitcnt lgkmcnt(0)`.
 
+A second rule of the same kind: a vector store of more than 8 bytes still reads its data registers for two cycles after
+it has issued.  The compiler inserts the wait states behind the stores it emits itself, but not behind one inside an
+inline-asm statement, where the next vector instruction may overwrite the data: such a store must be followed, inside
+its own statement, by `s_nop 1` or more.
+
 usage: check_sgpr_pipeline.py file.s [file.s ...]
 """
 import re
@@ -20,6 +25,8 @@ WAIT_ALL = re.compile(r"^\s*s_waitcnt\s+(0|0x0+)\s*$")
 SREG = re.compile(r"\bs(\d+)\b")
 SRANGE = re.compile(r"\bs\[(\d+):(\d+)\]")
 LABEL = re.compile(r"^[.\w$]+:")
+WIDE_STORE = re.compile(r"^\s*(global|buffer|flat|scratch)_store_dwordx[34]\b")
+NOP = re.compile(r"^\s*s_nop\s+(\d+)")
 
 
 def sregs_read(line):
@@ -43,6 +50,7 @@ def check(path):
     kernel = None
     in_asm = False
     in_flight = {}  # sgpr -> line number of the load
+    wide_store = None  # line number of a wide store in the current asm statement that still waits for its s_nop
     for no, line in enumerate(open(path), 1):
         text = line.rstrip("\n")
         if LABEL.match(text) and not text.startswith(".L"):
@@ -54,6 +62,21 @@ def check(path):
             continue
         if ";;#ASMEND" in text:
             in_asm = False
+            if wide_store is not None:
+                problems.append("%s:%d: a store of more than 8 bytes in inline asm without s_nop 1 behind it (kernel %s)" % (
+                    path, wide_store, kernel))
+                wide_store = None
+            continue
+        if in_asm and wide_store is not None:
+            m = NOP.match(text)
+            if not (m and int(m.group(1)) >= 1):
+                problems.append("%s:%d: a store of more than 8 bytes in inline asm without s_nop 1 behind it (kernel %s)" % (
+                    path, wide_store, kernel))
+            wide_store = None
+            if m:
+                continue
+        if in_asm and WIDE_STORE.match(text):
+            wide_store = no
             continue
         if WAIT0.match(text) or WAIT_ALL.match(text):
             in_flight.clear()

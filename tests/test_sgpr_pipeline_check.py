@@ -60,3 +60,31 @@ def test_checker_passes_the_pipeline_and_flags_a_spill_in_flight(tmp_path):
     # a copy to another SGPR or a use as a 64-bit pair operand is caught too
     bad.write_text(BAD.replace("v_writelane_b32 v57, s13, 22", "s_and_b64 vcc, exec, s[26:27]"))
     assert any("s_and_b64" in p for p in chk.check(str(bad)))
+
+
+def test_checker_wants_wait_states_behind_a_wide_store_in_inline_asm(tmp_path):
+    """A store of more than 8 bytes inside an inline-asm statement must carry its own `s_nop 1`: the compiler's hazard
+    handling does not see it, and the next vector instruction could overwrite the data it still reads."""
+    chk = load_checker()
+    good = tmp_path / "good.s"
+    good.write_text("""
+_Z6kernelv:
+	;;#ASMSTART
+	global_store_dwordx4 v[154:155], v[144:147], off sc1
+	s_nop 1
+	;;#ASMEND
+	v_mov_b32 v144, 1
+	;;#ASMSTART
+	global_store_dwordx2 v[154:155], v[144:145], off sc1
+	;;#ASMEND
+	global_store_dwordx4 v[2:3], v[4:7], off nt
+	s_endpgm
+""")
+    assert chk.check(str(good)) == []
+    for body in ("global_store_dwordx4 v[154:155], v[144:147], off sc1\n",
+                 "global_store_dwordx4 v[154:155], v[144:147], off sc1\n\ts_nop 0\n",
+                 "global_store_dwordx3 v[154:155], v[144:146], off\n\tv_mov_b32 v144, 1\n"):
+        bad = tmp_path / "bad.s"
+        bad.write_text("_Z6kernelv:\n\t;;#ASMSTART\n\t" + body + "\t;;#ASMEND\n\tv_mov_b32 v144, 1\n\ts_endpgm\n")
+        problems = chk.check(str(bad))
+        assert len(problems) == 1 and "more than 8 bytes" in problems[0], (body, problems)
