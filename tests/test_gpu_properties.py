@@ -63,6 +63,31 @@ def test_bconv_batch64_equals_float_convolution(dab, hw, cin, cout, stride):
     np.testing.assert_array_equal(cnt[17].cpu().numpy(), cpu)
 
 
+@pytest.mark.parametrize("n,h,w,cin,cout,stride", [
+    # outputs on both sides of the sizes at which a launch of raw counts starts to write through the L2 (6 MB with
+    # 32-channel staging windows, 9 MB with 16-channel ones), ragged pixel counts, channel counts that are no
+    # multiple of a window, every channel depth, both strides
+    (23, 31, 29, 64, 72, 1), (37, 30, 27, 64, 104, 1), (90, 41, 39, 64, 64, 2), (150, 29, 31, 64, 136, 2),
+    (21, 27, 25, 128, 136, 1), (35, 26, 29, 128, 152, 1), (61, 33, 31, 128, 200, 2),
+    (70, 15, 13, 256, 120, 1), (100, 14, 15, 256, 264, 1), (170, 17, 15, 256, 520, 2),
+    (111, 9, 7, 512, 232, 1), (190, 8, 9, 512, 520, 1), (45, 56, 56, 64, 64, 1),
+])
+def test_bconv_sizes_around_the_store_policy_switch(dab, n, h, w, cin, cout, stride):
+    """dab_bconv3x3 against the float convolution of the +-1 tensors (exact in fp32), whole tensor, at sizes where
+    the launcher changes the way the stores go through the L2 and where waves' ranges cut staging windows apart."""
+    gen = torch.Generator().manual_seed(n * 7 + h * 3 + cout)
+    x = rand_words(gen, n, h, w, cin // 64)
+    wt = rand_words(gen, cout, 9 * cin // 64)
+    cnt = dab.bconv_3x3(x, wt, stride, 1)
+    xs = unpack_pm1(x, cin).permute(0, 3, 1, 2)
+    ws = unpack_pm1(wt.reshape(cout, 3, 3, cin // 64), cin).permute(0, 3, 1, 2)
+    torch.backends.cudnn.allow_tf32 = False
+    torch.backends.cuda.matmul.allow_tf32 = False
+    conv = F.conv2d(F.pad(xs, (1, 1, 1, 1), value=-1.0), ws, stride=stride).permute(0, 2, 3, 1)
+    want = (9 * cin - conv) / 2
+    assert torch.equal(cnt, want), (cnt - want).abs().max().item()
+
+
 @pytest.mark.parametrize("hw,cin,cout,stride", [(56, 64, 64, 1), (14, 256, 256, 1), (28, 128, 256, 2)])
 def test_bconv_complement_symmetry(dab, hw, cin, cout, stride):
     gen = torch.Generator().manual_seed(99)
