@@ -73,6 +73,7 @@ SIGNATURES = {
     "dab_bconv3x3_splits_depth": (_i, [_i64, _i, _i]),
     "dab_bconv3x3_build": (_i, [_i64, _i, _i]),
     "dab_bconv3x3_counts_build": (_i, [_i64, _i, _i, _i]),
+    "dab_bconv3x3_epilogue_build": (_i, [_i64, _i, _i, _i, _i]),
     "dab_bconv3x3_fused_shares_tiles": (_i, [_i64, _i, _i]),
     "dab_prelu_inplace": (_i, [_vp, _i64, _i, _vp, _i, _vp]),
     "dab_concat_channels": (_i, [_vp, _i, _vp, _i, _i64, _vp, _vp]),

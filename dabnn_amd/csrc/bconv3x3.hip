@@ -249,11 +249,6 @@ __global__ __launch_bounds__(64 * kWavesPerBlock, (Residency<CW, NARROW>::waves_
 template <int CW, int MODE>
 __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
     typedef RowSplit<CW> RS;
-    // Raw counts only in the dispatch.  The store pass is written for every epilogue and the builds with one agree
-    // with the CPU layers on every case of the parity tests when they are forced onto them; against the other kernels
-    // they are behind at batch 1-4 with sign bits and at batch 256, and 5-30 % ahead between batch 8 and 64, which
-    // the dispatch (and the net's choice of who writes the sign bits) does not use yet.
-    static_assert(MODE == kModeCounts, "the row-split kernel is dispatched for raw counts only");
     constexpr int DWR = RS::row_dwords, VEC = RS::vec, PIECES = RS::pieces, GROUP = RS::group, SEG = RS::segment, ROW = RS::row;
     constexpr int kFilterBytes = 9 * CW * 8;  // one output channel's weights
     constexpr int kPixelBytes = CW * 8;
@@ -745,12 +740,22 @@ constexpr int kBuildSplitDepth = 0, kBuildWide = 1, kBuildNarrow = 2, kBuildRows
 // against 11.4 at batch 32, 15.7 against 17.0 at batch 64, 19.2 against 18.6 at batch 80, 30.0 against 27.7 at batch
 // 128; 14 x 14 x 256 -> 512 at stride 2: 3.1 against 3.8 us at batch 1, 4.7 against 6.1 at batch 16, 6.2 against 8.0 at
 // batch 32, 9.3 against 10.1 at batch 64, 11.4 against 11.1 at batch 80; 14 x 14 x 256 -> 256: 3.1 against 3.8 us at
-// batch 1, 6.0 against 7.0 at batch 16, 8.2 against 8.3 at batch 24, 11.4 against 9.9 at batch 40.  With an epilogue
-// the kernel is level or behind at most sizes (and with sign bits at every small one): raw counts only.
+// batch 1, 6.0 against 7.0 at batch 16, 8.2 against 8.3 at batch 24, 11.4 against 9.9 at batch 40.  The entry points
+// with an epilogue take it in a narrower window (below).
 static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode) {
-    if (mode != kModeCounts || cout % 8 != 0) return false;
-    if (cin == 512 || (cin == 256 && stride >= 2)) return tiles * cout <= 28ll * simd_count();
-    if (cin == 256) return tiles * cout <= 16ll * simd_count();
+    if (cout % 8 != 0 || !(cin == 512 || cin == 256)) return false;
+    const bool deep = cin == 512 || stride >= 2;  // 512 input channels, or 256 at stride 2
+    const long long work = tiles * cout, simds = simd_count();
+    if (mode == kModeCounts) return work <= (deep ? 28 : 16) * simds;
+    // With an epilogue the small-problem kernel stays ahead at small batches (its work items are whole bytes of sign
+    // bits and its first wave has the shortcut in flight from the start) and the unit kernel from mid-sized ones on;
+    // between them, measured at batches 1 to 64 of the three deep stage shapes: Affine + Add 7.8 against 8.2 us at
+    // batch 16 and 18.3 against 19.1 at batch 64 (7x7 512->512), 6.8 against 8.5 at batch 16 (14x14 256->256); with
+    // sign bits 14.3 against 19.9 us at batch 48 and 17.4 against 25.4 at batch 64 (7x7 512->512, where the unit
+    // kernel's work items of four units are coarse), 8.8 against 10.6 at batch 24 (14x14 256->256), 7.8 against 9.8 at
+    // batch 32 (14x14 256->512 at stride 2).
+    if (mode == kModeAffineAdd) return work >= 6 * simds && work <= (deep ? 28 : 16) * simds;
+    if (mode == kModeAffineAddSign) return cout % 64 == 0 && work >= (cin == 512 ? 8 : 6) * simds && work <= 28 * simds;
     return false;
 }
 
@@ -776,7 +781,7 @@ static int launch_bconv3x3(BconvArgs &a, long long tiles, hipStream_t stream) {
     }
     const int build = pick_build(tiles, CW * 64, a.cout, a.stride, MODE);
     if (build == kBuildSplitDepth) return launch_ksplit<CW, MODE>(a, tiles, stream);
-    if constexpr (CW >= 4 && MODE == kModeCounts) {
+    if constexpr (CW >= 4) {
         if (build == kBuildRows) return launch_rows<CW, MODE>(a, tiles, stream);
     }
     if (build == kBuildNarrow) return launch_variant<CW, MODE, true>(a, tiles, stream);
@@ -892,6 +897,12 @@ extern "C" int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout) {
     if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return -1;
     // the builds of the entry points with an epilogue; dab_bconv3x3_counts_build answers for dab_bconv3x3 itself
     return dab::pick_build((n_out_pixels + 63) / 64, cin, cout, 1, dab::kModeAffineAdd);
+}
+
+extern "C" int dab_bconv3x3_epilogue_build(int64_t n_out_pixels, int cin, int cout, int stride, int with_sign) {
+    if (n_out_pixels <= 0 || cout <= 0 || cout % 8 != 0 || stride <= 0 || !(cin == 64 || cin == 128 || cin == 256 || cin == 512)) return -1;
+    if (with_sign && cout % 64 != 0) return -1;
+    return dab::pick_build((n_out_pixels + 63) / 64, cin, cout, stride, with_sign ? dab::kModeAffineAddSign : dab::kModeAffineAdd);
 }
 
 extern "C" int dab_bconv3x3_counts_build(int64_t n_out_pixels, int cin, int cout, int stride) {

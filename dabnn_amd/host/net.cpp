@@ -370,11 +370,14 @@ void Net::fuse_binconv_epilogues() {
         if (!producer || !producer->fused_a || producer->output_mat->c % 64 != 0) continue;
         // not with 512 input channels: sign bits need work items of 8 output channels, four units there, and the
         // coarser split costs more than the separate pack_mat it saves (measured at batch 64 and 256) -- unless the
-        // problem is small enough for the kernel whose work items are 8 channels anyway
-        if (producer->input_mat->elem_c >= 512 &&
-            !dab_bconv3x3_splits_depth((int64_t)producer->output_mat->n * producer->output_mat->h * producer->output_mat->w,
-                                       producer->input_mat->elem_c, producer->output_mat->c))
-            continue;
+        // problem is small enough for the kernel whose work items are 8 channels anyway, or of the size that the
+        // row-split kernel takes (its store pass writes the bits at no extra pass)
+        if (producer->input_mat->elem_c >= 512) {
+            const int64_t pixels = (int64_t)producer->output_mat->n * producer->output_mat->h * producer->output_mat->w;
+            if (!dab_bconv3x3_splits_depth(pixels, producer->input_mat->elem_c, producer->output_mat->c) &&
+                dab_bconv3x3_epilogue_build(pixels, producer->input_mat->elem_c, producer->output_mat->c, producer->stride_h, 1) != 3)
+                continue;
+        }
         for (size_t j = i + 1; j < layers.size(); ++j) {
             auto consumer = std::dynamic_pointer_cast<BinConv>(layers[j]);
             if (consumer && consumer->input_mat == producer->output_mat) {

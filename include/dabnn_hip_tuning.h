@@ -33,12 +33,20 @@ DAB_API int dab_bconv3x3_splits_depth(int64_t n_out_pixels, int cin, int cout);
 DAB_API int dab_bconv3x3_build(int64_t n_out_pixels, int cin, int cout);
 
 /*
- * The same for dab_bconv3x3 itself (raw counts), which has a fourth build for mid-sized problems with 512 input
- * channels, or 256 at a stride of 2 or more: 3 = the row-split kernel, whose blocks are three waves that count one
- * kernel row each and add their partial counts in LDS.  dab_bconv3x3_build answers for the entry points with an
- * epilogue, which never take it.
+ * The same for dab_bconv3x3 itself (raw counts), which has a fourth build for 256 and 512 input channels from a
+ * single tile up to mid-sized problems: 3 = the row-split kernel, whose blocks are three waves that count one kernel
+ * row each and add their partial counts in LDS.  dab_bconv3x3_build answers for dab_bconv3x3_affine_add at stride 1
+ * and never says 3; dab_bconv3x3_epilogue_build knows stride and sign bits.
  */
 DAB_API int dab_bconv3x3_counts_build(int64_t n_out_pixels, int cin, int cout, int stride);
+
+/*
+ * The same for dab_bconv3x3_affine_add (with_sign = 0) and dab_bconv3x3_affine_add_sign (with_sign = 1) at a given
+ * stride: 0, 1, 2 as dab_bconv3x3_build names them, 3 = the row-split kernel, which these entry points take for 256
+ * and 512 input channels between the small and the mid-sized problems.  Net::prepare asks it for producers with 512
+ * input channels: where the answer is 3, the packed copy for the next binary convolution costs no separate pass.
+ */
+DAB_API int dab_bconv3x3_epilogue_build(int64_t n_out_pixels, int cin, int cout, int stride, int with_sign);
 
 /*
  * Whether dab_bconv3x3_affine_add(_sign) runs a problem of n_out_pixels = N*OH*OW on

@@ -19,7 +19,7 @@ def test_dispatch_probes_live_in_the_tuning_header():
     """dabnn_hip.h is the reference's surface plus the documented extensions; the probes that only say which kernel
     would run are declared in dabnn_hip_tuning.h."""
     probes = declared_symbols(("dabnn_hip_tuning.h",))
-    assert probes == sorted(["dab_bconv3x3_build", "dab_bconv3x3_counts_build", "dab_bconv3x3_splits_depth", "dab_bconv3x3_fused_shares_tiles",
+    assert probes == sorted(["dab_bconv3x3_build", "dab_bconv3x3_counts_build", "dab_bconv3x3_epilogue_build", "dab_bconv3x3_splits_depth", "dab_bconv3x3_fused_shares_tiles",
                              "dab_global_ave_pool_fconv1x1_takes", "dab_fconv_maxpool_pays"])
     assert not set(probes) & set(declared_symbols(("dabnn_hip.h",)))
 

@@ -324,13 +324,49 @@ def test_row_split_kernel_counts(dab, n, h, w, cin, cout, stride, pad):
     got = dab.bconv_3x3(dev_u(x), dev_u(wgt), stride, pad).cpu().numpy()
     want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, pad, pad, stride, stride) for img in x])
     np.testing.assert_array_equal(got, want)
-    # the entry points with an epilogue stay on the other builds and agree with it
+    # the entry point with an epilogue (on whichever build it takes at this size) agrees with it
     a = (r.standard_normal(cout) / 50).astype(np.float32)
     b = r.standard_normal(cout).astype(np.float32)
     fused = dab.bconv_3x3_affine_add(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), None, stride, pad)
     sep = dev_f(want.copy())
     dab.affine_inplace(sep, dev_f(a), dev_f(b))
     assert torch.equal(fused, sep)
+
+
+@pytest.mark.parametrize("n,h,w,cin,cout,stride,with_shortcut", [
+    # the sizes between the small and the mid-sized problems at which the entry points with an epilogue take the
+    # row-split kernel: the deep stage shapes of Bi-Real-18 at batch 16 to 64, a ragged pixel count, no shortcut
+    (32, 7, 7, 512, 512, 1, True), (64, 7, 7, 512, 512, 1, True), (16, 14, 14, 256, 256, 1, True),
+    (24, 14, 14, 256, 512, 2, True), (50, 9, 7, 512, 192, 1, False), (21, 13, 15, 256, 320, 1, True),
+])
+def test_fused_epilogues_through_the_row_split_kernel(dab, n, h, w, cin, cout, stride, with_shortcut):
+    """BinConv + Affine + Add (+ sign) through the row-split kernel, named by the library: the fp32 result against the
+    three reference layers and the packed copy against pack_mat of it, bit for bit, whole batch."""
+    from dabnn_amd import capi
+    oh, ow = (h + 2 - 3) // stride + 1, (w + 2 - 3) // stride + 1
+    assert capi.lib.dab_bconv3x3_epilogue_build(n * oh * ow, cin, cout, stride, 1) == 3
+    r = rng(41)
+    cw = cin // 64
+    x = r.integers(0, 2**64, size=(n, h, w, cw), dtype=np.uint64)
+    wgt = r.integers(0, 2**64, size=(cout, 9 * cw), dtype=np.uint64)
+    a = (r.standard_normal(cout) / 50).astype(np.float32)
+    b = r.standard_normal(cout).astype(np.float32)
+    a[::5] = 0.0
+    b[::10] = 0.0
+    want = np.stack([orc.baseline_bconv(img, wgt, 3, 3, 1, 1, stride, stride) for img in x])
+    sc = r.standard_normal(want.shape).astype(np.float32) if with_shortcut else None
+    for img in want:
+        orc.affine_inplace(img, a, b)
+    if with_shortcut:
+        sc[:, :, :, ::10] = 0.0
+        want = want + sc
+    got, packed = dab.bconv_3x3_affine_add_sign(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b),
+                                                dev_f(sc) if with_shortcut else None, stride, 1)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    np.testing.assert_array_equal(host_u(packed), np.stack([orc.pack_mat(img) for img in want]))
+    if capi.lib.dab_bconv3x3_epilogue_build(n * oh * ow, cin, cout, stride, 0) == 3:
+        plain = dab.bconv_3x3_affine_add(dev_u(x), dev_u(wgt), dev_f(a), dev_f(b), dev_f(sc) if with_shortcut else None, stride, 1)
+        np.testing.assert_array_equal(plain.cpu().numpy(), want)
 
 
 @pytest.mark.parametrize("n,h,w,cin,cout,stride,build", [

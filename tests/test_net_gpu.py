@@ -191,11 +191,18 @@ def test_bireal18_batch2_matches_cpu(mods, tmp_path, stem, batch):
     report = n.time_report()
     assert "Bin Conv" in report and "Float Conv" in report and "total" in report
     n.close()
-    # at a larger batch the two producers with 512 input channels leave the packing to their successors
-    big = net.Net(batch=64).read(str(path))
-    descs = big.layers()
+    # at a large batch the two producers with 512 input channels leave the packing to their successors (the unit
+    # kernel's work items of four units make the sign bits dearer than a separate pass there) ...
+    large = net.Net(batch=256).read(str(path))
+    descs = large.layers()
     assert sum("+ Sign" in d for d in descs if d.startswith("Bin Conv")) == 13
     assert sum("packed input from its producer" in d for d in descs) == 14
+    large.close()
+    # ... and write them themselves at the sizes the row-split kernel takes
+    big = net.Net(batch=64).read(str(path))
+    descs = big.layers()
+    assert sum("+ Sign" in d for d in descs if d.startswith("Bin Conv")) == 15
+    assert sum("packed input from its producer" in d for d in descs) == 16
     # and either stem's last convolution runs with its MaxPool inside (the three-convolution stem's on the
     # split-operand kernel at this size, which pools a tile column's rows and columns in registers)
     assert sum("+ MaxPool 3x3 stride 2 + Sign" in d for d in descs) == 1
