@@ -762,14 +762,30 @@ static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode)
 static int pick_build(long long tiles, int cin, int cout, int stride = 1, int mode = kModeCounts) {
     if (takes_rows(tiles, cin, cout, stride, mode)) return kBuildRows;
     if (splits_depth(tiles, cin, cout)) return kBuildSplitDepth;
+    const long long simds = simd_count();
     if (cin <= 128) {
-        // four (eight) units or more per wave at four waves per SIMD
         const long long units = tiles * (cout / 8);
-        if (units >= (cin == 64 ? 4ll : 8ll) * simd_count() * 4) return kBuildNarrow;
+        if (mode != kModeCounts) {
+            // with an epilogue: four (eight) units or more per wave at four waves per SIMD
+            if (units >= (cin == 64 ? 4ll : 8ll) * simds * 4) return kBuildNarrow;
+        } else if (cin == 64) {
+            // Raw counts, whose stores are written through and whose 64-byte runs then cost nothing extra: the
+            // four-wave build is ahead only at stride 1 between 24 and 44 units per SIMD (56x56 64->64: 12.5 against
+            // 11.4 us at batch 48, 14.7 against 15.1 at batch 64, 20.0 against 20.5 at batch 96; 27.9 against 26.5 at batch 128, 52.2 against 49.8
+            // at batch 256; 56x56 64->128 at stride 2: 12.4 against 11.5 at batch 96, 27.8 against 26.1 at batch 256)
+            if (stride == 1 && units >= 24 * simds && units < 44 * simds) return kBuildNarrow;
+        } else {
+            // 128 input channels: from 16 units per SIMD at stride 1 (28x28 128->128: 18.4 against 20.1 us at batch
+            // 96, 22.9 against 24.2 at batch 128, level at batch 64), from 4 at stride 2 (28x28 128->256: 7.6
+            // against 8.7 us at batch 48, 23.0 against 24.6 at batch 256)
+            if (units >= (stride >= 2 ? 4 : 16) * simds) return kBuildNarrow;
+        }
     } else {
-        // six large units or more per wave
+        // large units: six or more per wave; raw counts with 512 input channels from three (7x7 512->512: 21.3 against
+        // 21.9 us at batch 96, 26.4 against 27.8 at batch 128)
         const long long big_units = tiles * (cout / (cin == 256 ? 8 : 4));
-        if (cout % 8 == 0 && big_units >= 6ll * simd_count() * (cin == 256 ? 4 : 3)) return kBuildNarrow;
+        const long long per_wave = (mode == kModeCounts && cin == 512) ? 3 : 6;
+        if (cout % 8 == 0 && big_units >= per_wave * simds * (cin == 256 ? 4 : 3)) return kBuildNarrow;
     }
     return kBuildWide;
 }
