@@ -322,21 +322,6 @@ __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
             __syncthreads();
         }
 
-        // the whole-segment store pass's shortcut values, asked for before the counting so that they arrive behind it
-        float4 sc_pre[3];
-        bool pre_ok = false;
-        if constexpr (MODE == kModeAffineAdd || MODE == kModeAffineAddSign) {
-            if (p.epi_shortcut != nullptr && seg == SEG && (tile + 1) * 64 <= p.total) {
-                pre_ok = true;
-#pragma unroll
-                for (int j = 0; j < 3; ++j) {
-                    const int pr = (tid >> 3) + j * (RS::threads / 8);
-                    sc_pre[j] = pr < 64 ? *reinterpret_cast<const float4 *>(p.epi_shortcut + ((size_t)tile * 64 + pr) * p.cout + cbase + (tid & 7) * 4)
-                                        : make_float4(0.f, 0.f, 0.f, 0.f);
-                }
-            }
-        }
-
         {
             // this wave's weights: row r of the segment's channels, GROUP channels per pass.  The scalar-load batches
             // form one sequence (channel by channel, PIECES per channel) and batch j lives in wv[j & 1]: the one a body
@@ -377,14 +362,14 @@ __global__ __launch_bounds__(192) void bconv3x3_rows_kernel(const BconvArgs p) {
             EpiAffineAddSign epi;
             epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
             epi.bits = p.epi_bits, epi.bits_ld = p.cout >> 3;
-            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi);
         } else if constexpr (MODE == kModeAffineAdd) {
             EpiAffineAdd epi;
             epi.a = p.epi_a, epi.b = p.epi_b, epi.shortcut = p.epi_shortcut;
-            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi);
         } else {
             EpiStore epi;
-            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi, sc_pre, pre_ok);
+            rows_flush<SEG, ROW, RS::threads>(plane, tid, p.out, p.cout, tile, p.total, cbase, seg, epi);
         }
         left -= seg, ch += seg;
         if (ch == p.cout) ch = 0, ++tile;

@@ -10,8 +10,7 @@
 // (48 or 24 dwords) and reach v_xor_b32 as SGPR operands from scalar loads, as in the unit kernel: per 32 bits of
 // depth and per output one v_xor_b32 and one v_bcnt_u32_b32.  The three partial counts of an output meet in LDS
 // (ds_add_u32 on a plane of 64 pixels x 32 channels that starts at zero and that the store pass leaves at zero), and
-// the block writes the plane out in 16-byte parts through the epilogue: whole 128-byte lines per pixel for a full
-// segment.
+// the block writes the plane out in 16-byte parts through the epilogue.
 //
 // Work split: a block owns a contiguous range of output channels over the tiles of 64 pixels, cut at multiples of
 // four channels (eight when sign bits are written), and walks it in segments of at most 32 channels of one tile.
@@ -85,13 +84,15 @@ __device__ __forceinline__ void rows_count(uint32_t &acc, const WVec<DW> &w, con
 }
 
 // The store pass of a block: the plane's channels [0, seg) of a tile of 64 pixels go to out[pixel][cbase + ...]
-// through the epilogue, and the plane is left at zero.  seg is a multiple of 4 (of 8 when sign bits are written).
-// sc_pre: the shortcut values of the whole-segment pass, fetched by the caller before it counted.
+// through the epilogue, in 16-byte parts (four channels), and the plane is left at zero.  seg is a multiple of 4 (of 8
+// when sign bits are written).  A block's share is at most 24 channels wherever the launcher takes this kernel (at most
+// 28 channel-tiles per SIMD over six blocks per CU), so the parts of a pixel are a piece of a line whose rest another
+// block writes at another time: they are written through the L2 at device scope.  As ordinary or streaming stores
+// the pieces wait in the L2 for the rest of their line; 14x14 256->512 at stride 2: 6.1 against 7.9 us at batch 32,
+// 9.15 against 9.7 at batch 64; 7x7 512->512 at batch 64: 15.7 against 16.6.
 template <int SEG, int ROW, int THREADS, class Epi>
 __device__ __forceinline__ void rows_flush(unsigned char *plane, int tid, float *__restrict__ out, int ld, int tile, int total,
-                                           int cbase, int seg, Epi epi, const float4 (&sc_pre)[3], bool pre_ok) {
-    constexpr int NP = SEG / 4;  // 16-byte parts per pixel row of a whole segment
-    static_assert(NP == 8 && THREADS % NP == 0, "eight lanes to a pixel");
+                                           int cbase, int seg, Epi epi) {
     typedef float f32x4 __attribute__((ext_vector_type(4)));
     // per-thread offsets of the pass are loop invariants of the caller: derived from an index the compiler cannot see
     // through they are made here and do not live across the counting
@@ -99,88 +100,40 @@ __device__ __forceinline__ void rows_flush(unsigned char *plane, int tid, float 
     const bool has_sc = Epi::kShortcut && epi.shortcut != nullptr;
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
     auto to_float = [](u32x4 c) { return make_float4((float)c.x, (float)c.y, (float)c.z, (float)c.w); };
-    if (seg == SEG && (tile + 1) * 64 <= total) {
-        const int part = tid & (NP - 1);
-        epi.prepare(cbase + part * 4);
-        auto round = [&](int j, const float4 &sc_j) {
-            const int pr = tid / NP + j * (THREADS / NP);  // 24 pixels per round: 24, 24, 16
-            uint32_t w = 0;
-            if (pr < 64) {
-                u32x4 *src = reinterpret_cast<u32x4 *>(plane + pr * ROW + part * 16);
-                const float4 v = to_float(*src);
-                *src = zero4;
-                const size_t off = ((size_t)tile * 64 + pr) * ld + cbase + part * 4;
+    const int np = seg >> 2;                  // 16-byte parts per pixel row
+    const int magic = (65536 + np - 1) / np;  // c / np for c < 512
+    const int rounds = (64 * np + THREADS - 1) / THREADS;
+    static_assert(SEG <= 32, "64 * SEG / 4 part indices stay below 512");
+    // every thread makes the same number of rounds (the sign bytes are gathered across lanes)
+    for (int i = 0; i < rounds; ++i) {
+        const int c = tid + i * THREADS;
+        const bool in_plane = c < 64 * np;
+        const int pr = in_plane ? (c * magic) >> 16 : 0;
+        const int part = in_plane ? c - pr * np : 0;
+        const int pix = tile * 64 + pr;
+        uint32_t nib = 0;
+        if (in_plane) {
+            u32x4 *src = reinterpret_cast<u32x4 *>(plane + pr * ROW + part * 16);
+            const float4 v = to_float(*src);
+            *src = zero4;
+            if (pix < total) {
+                const size_t off = (size_t)pix * ld + cbase + part * 4;
+                epi.prepare(cbase + part * 4);
                 float4 r;
-                if (has_sc) {
-                    const float4 sc = pre_ok ? sc_j
-                                             : *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off);
-                    r = epi.template apply<Epi::kShortcut>(v, sc);
-                } else {
+                if (has_sc)
+                    r = epi.template apply<Epi::kShortcut>(
+                        v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
+                else
                     r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
-                }
-                // streaming store: the output is not read again by this kernel
-                __builtin_nontemporal_store(f32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<f32x4 *>(out + off));
-                if constexpr (Epi::kEmit) w = sign_nibble(r) << (4 * part);
+                store_through(reinterpret_cast<f32x4 *>(out + off), f32x4{r.x, r.y, r.z, r.w});
+                if constexpr (Epi::kEmit) nib = sign_nibble(r);
             }
-            if constexpr (Epi::kEmit) {
-                // the eight lanes of a pixel hold its segment's sign bits, four each: gather them in the first lane
-                w = or_from_lane_above<1>(w);
-                w = or_from_lane_above<2>(w);
-                w = or_from_lane_above<4>(w);
-                if (pr < 64 && part == 0)
-                    *reinterpret_cast<uint32_t *>(epi.bits + ((size_t)tile * 64 + pr) * epi.bits_ld + (cbase >> 3)) = w;
-            }
-        };
-        if constexpr (Epi::kShortcut) {
-            round(0, sc_pre[0]);
-            round(1, sc_pre[1]);
-            round(2, sc_pre[2]);
-        } else {
-            // rolled: the rounds' temporaries would otherwise all live beside the activation registers
-            const float4 none = make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll 1
-            for (int j = 0; j < 3; ++j) round(j, none);
         }
-    } else {
-        const int np = seg >> 2;                  // 16-byte parts per pixel row
-        const int magic = (65536 + np - 1) / np;  // c / np for c < 512
-        const int rounds = (64 * np + THREADS - 1) / THREADS;
-        // every thread makes the same number of rounds (the sign bytes are gathered across lanes)
-        for (int i = 0; i < rounds; ++i) {
-            const int c = tid + i * THREADS;
-            const int pr = (c * magic) >> 16;
-            const int part = c - pr * np;
-            const int pix = tile * 64 + pr;
-            const bool in_plane = c < 64 * np;
-            uint32_t nib = 0;
-            if (in_plane) {
-                u32x4 *src = reinterpret_cast<u32x4 *>(plane + pr * ROW + part * 16);
-                const float4 v = to_float(*src);
-                *src = zero4;
-                if (pix < total) {
-                    const size_t off = (size_t)pix * ld + cbase + part * 4;
-                    epi.prepare(cbase + part * 4);
-                    float4 r;
-                    if (has_sc)
-                        r = epi.template apply<Epi::kShortcut>(
-                            v, *reinterpret_cast<const float4 *>((Epi::kReadsOut ? const_cast<const float *>(out) : epi.shortcut) + off));
-                    else
-                        r = epi.template apply<false>(v, make_float4(0.f, 0.f, 0.f, 0.f));
-                    // Written through the L2 at device scope.  A block's share is 16 or 20 channels, so this is the
-                    // path nearly all of the kernel's output takes, in pieces of a line; as ordinary or streaming
-                    // stores the pieces wait in the L2 for the rest of their line, which another block writes at
-                    // another time.  14x14 256->512 at stride 2: 6.1 against 7.9 us at batch 32, 9.15 against 9.7 at
-                    // batch 64; 7x7 512->512 at batch 64: 15.7 against 16.6.
-                    store_through(reinterpret_cast<f32x4 *>(out + off), f32x4{r.x, r.y, r.z, r.w});
-                    if constexpr (Epi::kEmit) nib = sign_nibble(r);
-                }
-            }
-            if constexpr (Epi::kEmit) {
-                // np is even here and so are THREADS and 64 * np: the two halves of a byte sit in lanes 2k and 2k+1
-                uint32_t w = nib << (4 * (part & 1));
-                w = or_from_lane_above<1>(w);
-                if (in_plane && pix < total && !(part & 1)) epi.bits[(size_t)pix * epi.bits_ld + ((cbase + part * 4) >> 3)] = (unsigned char)w;
-            }
+        if constexpr (Epi::kEmit) {
+            // np is even here and so are THREADS and 64 * np: the two halves of a byte sit in lanes 2k and 2k+1
+            uint32_t w = nib << (4 * (part & 1));
+            w = or_from_lane_above<1>(w);
+            if (in_plane && pix < total && !(part & 1)) epi.bits[(size_t)pix * epi.bits_ld + ((cbase + part * 4) >> 3)] = (unsigned char)w;
         }
     }
 }
