@@ -739,7 +739,9 @@ static bool takes_rows(long long tiles, int cin, int cout, int stride, int mode)
     // sign bits 14.3 against 19.9 us at batch 48 and 17.4 against 25.4 at batch 64 (7x7 512->512, where the unit
     // kernel's work items of four units are coarse), 8.8 against 10.6 at batch 24 (14x14 256->256), 7.8 against 9.8 at
     // batch 32 (14x14 256->512 at stride 2).
-    if (mode == kModeAffineAdd) return work >= 6 * simds && work <= (deep ? 28 : 16) * simds;
+    // (without sign bits its work items are four channels, twice as many blocks as the small-problem kernel has: ahead
+    // again on one or two tiles, 4.6 against 5.1 us for one image of 7x7 512->512)
+    if (mode == kModeAffineAdd) return work <= simds || (work >= 6 * simds && work <= (deep ? 28 : 16) * simds);
     if (mode == kModeAffineAddSign) return cout % 64 == 0 && work >= (cin == 512 ? 8 : 6) * simds && work <= 28 * simds;
     return false;
 }
