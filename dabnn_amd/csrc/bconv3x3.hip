@@ -563,8 +563,8 @@ static int launch_variant(BconvArgs &a, long long tiles, hipStream_t stream) {
     return DAB_OK;
 }
 
-// Blocks per CU of the row-split kernel: six (18 waves) measured best at batch 64 (7 x 7 x 512 -> 512: 16.4 us with 6 to
-// 10, 17.2 with 4; 14 x 14 x 256 -> 512 at stride 2: 9.9 us with 6, 10.3-10.6 with 7 to 10).
+// Blocks per CU of the row-split kernel: six (18 waves) at least (7 x 7 x 512 -> 512 at batch 64: 16.8 us with 4,
+// 16.6 with 5, 15.7 with 6); launch_rows may take more for raw counts.
 constexpr int kRowsBlocksPerCu = 6;
 
 template <int CW, int MODE>
@@ -574,8 +574,27 @@ static int launch_rows(BconvArgs &a, long long tiles, hipStream_t stream) {
     const long long items = tiles * a.n_groups;
     if (items >= (1ll << 31) / a.gran) return fail(DAB_EUNSUPPORTED, "dab_bconv3x3: too many work units");
     static const int blocks_per_cu = resident_blocks_per_cu(bconv3x3_rows_kernel<CW, MODE>, RowSplit<CW>::threads);
-    const int per_cu = blocks_per_cu < kRowsBlocksPerCu ? blocks_per_cu : kRowsBlocksPerCu;
-    long long blocks = (long long)(simd_count() / 4) * per_cu;
+    // Blocks per CU.  A launch is one round of resident blocks, and it ends with its most loaded SIMD: the waves a
+    // SIMD holds (three per block over four SIMDs) times the items of the largest block plus one (what a block does
+    // before its first item -- activations, the plane -- is about an item's worth).  Raw counts take the count
+    // between six per CU (fewer waves issue their pairs more slowly) and what is resident (ten at most) with the
+    // smallest such product, the larger among equals (more waves hide more latency), as long as a block keeps two
+    // items.  Against a fixed six: 7x7 512->512 14.6 against 15.7 us at batch 64 (nine blocks per CU), 11.9 against
+    // 13.0 at batch 48; 14x14 256->512 at stride 2 7.6 against 8.2 at batch 48; level up to batch 28.  With an
+    // epilogue the same rule gained and lost up to 1.5 us from size to size: six.
+    const long long cus = simd_count() / 4;
+    int per_cu = blocks_per_cu < kRowsBlocksPerCu ? blocks_per_cu : kRowsBlocksPerCu;
+    if (MODE == kModeCounts) {
+        long long best = -1;
+        const int hi = blocks_per_cu < 10 ? blocks_per_cu : 10;
+        for (int c = kRowsBlocksPerCu < hi ? kRowsBlocksPerCu : hi; c <= hi; ++c) {
+            const long long b = cus * c < items ? cus * c : items;
+            if (c > kRowsBlocksPerCu && (items + b - 1) / b < 2) break;
+            const long long load = ((3 * b + simd_count() - 1) / simd_count()) * ((items + b - 1) / b + 1);
+            if (best < 0 || load <= best) best = load, per_cu = c;
+        }
+    }
+    long long blocks = cus * per_cu;
     if (blocks > items) blocks = items;
     a.items_per_wave = (int)(items / blocks);
     a.items_extra = (int)(items % blocks);
