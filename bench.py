@@ -32,12 +32,12 @@ BATCH = 64
 # HBM traffic of the headline workload per kernel launch (bytes, mean of the seven shapes), measured with
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on `bench.py --profile-mode` (summary: profiles/bconv3x3_config3_b64.md),
 # next to the algorithmic bytes (packed input + weights + fp32 output).
-TRAFFIC_BYTES_PER_LAUNCH = 24.80e6
+TRAFFIC_BYTES_PER_LAUNCH = 25.38e6
 ALGORITHMIC_BYTES_PER_LAUNCH = 21.10e6
 # where the constant comes from: it is not measured by this run (the counters need rocprofv3 around the process) and
 # goes stale when the kernel changes, so the profile and the kernel sources it was collected on are named with it
 TRAFFIC_SOURCE = ("profiles/bconv3x3_config3_b64.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on "
-                  "`bench.py --profile-mode`), collected on dabnn_amd/csrc/bconv3x3.hip + bconv3x3_rows.h + xnor_core.h as of commit f127f18")
+                  "`bench.py --profile-mode`), collected on dabnn_amd/csrc/bconv3x3.hip + bconv3x3_rows.h + xnor_core.h as of commit 10161d5")
 
 
 def out_dim(size, pad, k, stride):
