@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
                 sum = sum + a_reg[i][3];
                 v = sum * 0.25f;
                 const int pix = m0 + l_r + RP * i, k = k0 + CV * l_k;
-                if (blockIdx.y == 0 && pix < p.M && k < p.K)
+                if (p.pooled != nullptr && blockIdx.y == 0 && pix < p.M && k < p.K)
                     *reinterpret_cast<f32xcv *>(p.pooled + (size_t)pix * p.K + k) = v;
             }
 #pragma unroll
@@ -328,6 +328,179 @@ __global__ __launch_bounds__(256) void fconv_kernel(const FconvArgs p) {
         case 5: emit_all(T{}, F{}, T{}); break;
         case 6: emit_all(T{}, T{}, F{}); break;
         default: emit_all(T{}, T{}, T{}); break;
+    }
+}
+
+// AvePool 2x2 stride 2 + 1x1 convolution over K input channels (a multiple of 64; built for 64) when the launch is
+// bound by the input it reads.  fconv_kernel<..., POOL> pools a tile's pixels once per column tile and fetches a
+// pixel's channels slice by slice.  Here a block pools its BM pixels once, whole pixels at a time (4K contiguous bytes
+// per window pixel), into an LDS tile that holds all K depths, and walks the column tiles of 128 output channels over
+// it while the filters stream through a double buffer in slices of 32 depths.  Every sum takes its depths in the
+// order fconv_kernel takes them (eight at a time, the pairs d and d + 4 in one matrix instruction), so the results
+// are the same bit for bit.  p.pooled may be null: then the pooled tensor is not written.
+template <int K, int BM>
+__global__ __launch_bounds__(256) void pool2_fconv1x1_kernel(const FconvArgs p) {
+    constexpr int BN = 128, SK = 32, RS = SK + 4, AS = K + 4;  // row strides of 4 mod 64 floats: no bank conflicts
+    constexpr int THREADS = 256, WAVES_M = BM / 32, WAVES_N = 4 / WAVES_M, WTN = BN / WAVES_N, TN = WTN / 32;
+    constexpr int KV = K / 4;           // 16-byte pieces of a pixel
+    constexpr int A4 = BM * KV / THREADS;   // pieces of the pooled tile per thread
+    constexpr int AB = A4 < 4 ? A4 : 4;  // of which this many are in flight at a time (four loads each)
+    constexpr int SLICES = K / SK;
+    static_assert(BM == 32 || BM == 64, "one or two rows of waves");
+    constexpr int BJ = BN * 8 / THREADS;  // 16-byte pieces of a filter slice per thread
+    static_assert(K % SK == 0 && (BM * KV) % THREADS == 0 && A4 % AB == 0 && TN >= 1, "tile");
+    __shared__ __attribute__((aligned(16))) float As[BM][AS];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BN][RS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int m0 = blockIdx.x * BM;
+    const int img0 = (int)p.div_oh.div(p.div_ow.div((uint32_t)m0));
+    const int img_elems = p.h * p.wd * K;
+    const long long x_left = (long long)(p.n - img0) * img_elems * 4;
+    const auto x_rsrc = make_rsrc(p.x + (size_t)img0 * img_elems, (uint32_t)(x_left < kOobRow ? x_left : kOobRow));
+    const auto w_rsrc = make_rsrc(p.w, (uint32_t)p.cout * K * 4u);
+    const int rows_m = p.M - m0 < BM ? p.M - m0 : BM;
+    const auto o_rsrc = make_rsrc(p.out + (size_t)m0 * p.cout, (uint32_t)rows_m * p.cout * 4u);
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    auto load4 = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off) -> f32x4 {
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0));
+    };
+
+    // filters: slice `it` = column tile it / SLICES, depths 32 * (it % SLICES) ...; thread = 16 bytes of four rows
+    const int b_k = tid & 7, b_r = tid >> 3;
+    constexpr int BR = THREADS / 8;  // filter rows per pass of the block
+    const int tiles_n = (p.cout + BN - 1) / BN, total = tiles_n * SLICES;
+    // two slices ahead, through registers: a slice is asked for two iterations before it is multiplied (the first
+    // touch of a slice by any block comes from memory) and goes to the LDS buffer that the iteration before it freed
+    f32x4 b_reg[2][BJ];
+    auto fetch_b = [&](int it, int slot) {
+        const int nt = it / SLICES, ks = it - nt * SLICES;
+#pragma unroll
+        for (int j = 0; j < BJ; ++j) {
+            const int row = nt * BN + b_r + BR * j;
+            b_reg[slot][j] = load4(w_rsrc, row < p.cout ? (uint32_t)((row * K + ks * SK + 4 * b_k) * 4) : kOob);
+        }
+    };
+    auto commit_b = [&](int slot) {
+#pragma unroll
+        for (int j = 0; j < BJ; ++j) *reinterpret_cast<f32x4 *>(&Bs[slot][b_r + BR * j][4 * b_k]) = b_reg[slot][j];
+    };
+    fetch_b(0, 0);
+    if (total > 1) fetch_b(1, 1);
+
+    // the pooled tile: ave_pool_fallback (dabnn/layers/AvePool.cpp:84-123) for a 2x2 window without padding, the taps
+    // added to zero in row-major order and divided by 4 (a multiplication by 0.25 rounds the same way)
+    {
+        const uint32_t right = (uint32_t)K * 4u, below = (uint32_t)p.wd * right;
+#pragma unroll
+        for (int i0 = 0; i0 < A4; i0 += AB) {
+            f32x4 win[AB][4];
+#pragma unroll
+            for (int i = 0; i < AB; ++i) {
+                const int piece = tid + THREADS * (i0 + i), r = piece / KV, c4 = piece % KV;
+                const int pix = m0 + r;
+                const uint32_t t0 = p.div_ow.div((uint32_t)pix);
+                const int ox = pix - (int)t0 * p.ow, img = (int)p.div_oh.div(t0), oy = (int)t0 - img * p.oh;
+                const uint32_t off =
+                    pix < p.M ? (uint32_t)((((img - img0) * p.h + 2 * oy) * p.wd + 2 * ox) * K + 4 * c4) * 4u : kOobRow;
+                win[i][0] = load4(x_rsrc, off);
+                win[i][1] = load4(x_rsrc, off + right);
+                win[i][2] = load4(x_rsrc, off + below);
+                win[i][3] = load4(x_rsrc, off + below + right);
+            }
+#pragma unroll
+            for (int i = 0; i < AB; ++i) {
+#pragma clang fp contract(off)
+                const int piece = tid + THREADS * (i0 + i), r = piece / KV, c4 = piece % KV;
+                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+                sum = sum + win[i][0];
+                sum = sum + win[i][1];
+                sum = sum + win[i][2];
+                sum = sum + win[i][3];
+                const f32x4 v = sum * 0.25f;
+                *reinterpret_cast<f32x4 *>(&As[r][4 * c4]) = v;
+                if (p.pooled != nullptr && m0 + r < p.M)
+                    __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(p.pooled + (size_t)(m0 + r) * K + 4 * c4));
+            }
+        }
+    }
+    commit_b(0);
+    __syncthreads();
+
+    const uint32_t row_bytes = (uint32_t)p.cout * 4u;
+    const int f_k = lane >> 5, f_i = lane & 31;
+    // accumulator element e of lane l: row 8*(e/4) + 4*(l/32) + e%4, column l % 32
+    auto emit_tile = [&](auto has_bias, auto has_affine, auto has_relu, int n0, const f32x16 (&acc)[TN]) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int co = n0 + wn * WTN + j * 32 + f_i;
+            const bool co_ok = co < p.cout;
+            const float bias = (decltype(has_bias)::value && co_ok) ? p.bias[co] : 0.f;
+            const float fa = (decltype(has_affine)::value && co_ok) ? p.aff_a[co] : 0.f;
+            const float fb = (decltype(has_affine)::value && co_ok) ? p.aff_b[co] : 0.f;
+            const uint32_t lane_off = (co_ok ? (uint32_t)co * 4u : kOob) + (uint32_t)(wm * 32 + 4 * f_k) * row_bytes;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+#pragma clang fp contract(off)
+                float v = acc[j][e];
+                if constexpr (decltype(has_bias)::value) v = v + bias;
+                if constexpr (decltype(has_affine)::value) {
+                    const float prod = fa * v;
+                    v = prod + fb;
+                }
+                if constexpr (decltype(has_relu)::value) v = v < 0.f ? 0.f : v;  // std::max(v, 0.f): a NaN stays
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), o_rsrc,
+                                                      (int)(lane_off + (uint32_t)(8 * (e / 4) + (e % 4)) * row_bytes), 0, 0);
+            }
+        }
+    };
+    using T = std::true_type;
+    using F = std::false_type;
+    const int epilogue = (p.bias ? 4 : 0) | (p.aff_a ? 2 : 0) | (p.relu ? 1 : 0);
+
+    static_assert(SLICES % 2 == 0, "a slice's buffer is its number modulo 2 in every column tile");
+    f32x16 acc[TN];
+    for (int nt = 0; nt < tiles_n; ++nt) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < SLICES; ++ks) {
+            const int it = nt * SLICES + ks;
+            if (it + 2 < total) fetch_b(it + 2, ks & 1);
+#pragma unroll
+            for (int g = 0; g < SK / 8; ++g) {
+                const int kb = g * 8 + f_k * 4;
+                const float4 a4 = *reinterpret_cast<const float4 *>(&As[wm * 32 + f_i][ks * SK + kb]);
+                float4 b4[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    b4[j] = *reinterpret_cast<const float4 *>(&Bs[ks & 1][wn * WTN + j * 32 + f_i][kb]);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.x, b4[j].x, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.y, b4[j].y, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.z, b4[j].z, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a4.w, b4[j].w, acc[j], 0, 0, 0);
+                }
+            }
+            if (ks == SLICES - 1) {
+                switch (epilogue) {
+                    case 0: emit_tile(F{}, F{}, F{}, nt * BN, acc); break;
+                    case 1: emit_tile(F{}, F{}, T{}, nt * BN, acc); break;
+                    case 2: emit_tile(F{}, T{}, F{}, nt * BN, acc); break;
+                    case 3: emit_tile(F{}, T{}, T{}, nt * BN, acc); break;
+                    case 4: emit_tile(T{}, F{}, F{}, nt * BN, acc); break;
+                    case 5: emit_tile(T{}, F{}, T{}, nt * BN, acc); break;
+                    case 6: emit_tile(T{}, T{}, F{}, nt * BN, acc); break;
+                    default: emit_tile(T{}, T{}, T{}, nt * BN, acc); break;
+                }
+            }
+            // the other buffer was last read before the barrier that ended the previous slice
+            if (it + 1 < total) commit_b((ks + 1) & 1);
+            __syncthreads();
+        }
     }
 }
 
@@ -793,7 +966,7 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
                                       dab_stream_t stream) {
     using namespace dab;
     const char *fn = "dab_ave_pool2_fconv1x1";
-    DAB_REQUIRE(x && wgt && pooled && out, "%s: null pointer", fn);
+    DAB_REQUIRE(x && wgt && out, "%s: null pointer", fn);
     DAB_REQUIRE(n > 0 && h >= 2 && w >= 2 && c > 0 && cout > 0, "%s: bad dimension (the input must hold a 2x2 window)", fn);
     DAB_REQUIRE((aff_a == nullptr) == (aff_b == nullptr), "%s: affine needs both coefficient vectors", fn);
     if (c % 4 != 0 ||
@@ -811,6 +984,7 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
         return fail(DAB_EUNSUPPORTED, "%s: tensor too large for 32-bit indexing", fn);
     a.M = (int)M;
     if (M <= 8 && cout >= 64) {
+        DAB_REQUIRE(pooled, "%s: eight pooled pixels or fewer run as two launches and need the pooled tensor's buffer", fn);
         // a handful of pooled pixels: dab_fconv_affine_relu makes them with its matrix-vector kernel, whose sums are
         // added in another order than a tile's -- two launches, so that the result stays what the two calls give
         int rc = dab_ave_pool(x, n, h, w, c, 2, 2, 0, 0, 2, 2, pooled, stream);
@@ -831,7 +1005,17 @@ extern "C" int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c
                        dim3((unsigned)((M + BM - 1) / BM), (unsigned)((cout + BN - 1) / BN)), dim3(256), 0, s, a)
     // the same tiles as dab_fconv_affine_relu takes for the 1x1 convolution of the pooled tensor: the sums of a tile
     // whose depth is split over waves are added in another order
-    if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 1)
+    const bool few = big_tiles < simd_count() / 4;
+    const int small = few ? small_1x1_tiles(1, M, cout) : 0;
+    const bool depth_split = few && (small == 3 || (small == 0 && ((M + 63) / 64) * ((cout + 63) / 64) < simd_count() / 8));
+    if (c == 64 && cout > 64 && !depth_split && (long long)cout * c * 4 < (1ll << 30))
+        // 64 input channels: the launch is bound by the input it reads, and the kernel that pools whole pixels once
+        // into LDS reads it at the rate of a copy (256 x 56 x 56 x 64 -> 128: 66 us against 85, 58 without the pooled
+        // tensor; batch 8: 5.2 against 6.1).  With 128 and 256 channels the two forms take the same time at batch
+        // 256 (50 / 50 and 50 / 46 us), both at half of what the fp32 matrix instructions could do, and the tile
+        // kernel wins below.
+        hipLaunchKernelGGL((pool2_fconv1x1_kernel<64, 32>), dim3((unsigned)((M + 31) / 32)), dim3(256), 0, s, a);
+    else if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 1)
         DAB_POOLED_LAUNCH(64, 128, 32, 1);
     else if (big_tiles < simd_count() / 4 && small_1x1_tiles(1, M, cout) == 2)
         DAB_POOLED_LAUNCH(64, 64, 32, 1);

@@ -241,7 +241,7 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
         reads = {fc->fused_pool_input ? fc->fused_pool_input.get() : fc->input_mat.get()};
         writes = {fc->output_mat ? fc->output_mat.get() : fc->fused_maxpool_out.get()};
         if (fc->fused_maxpool_sign) writes.push_back(fc->fused_maxpool_sign.get());
-        if (fc->fused_pool_input) writes.push_back(fc->input_mat.get());  // the pooled blob, a side product
+        if (fc->fused_pool_input && fc->input_mat->dev) writes.push_back(fc->input_mat.get());  // the pooled blob, a side product
     } else if (auto af = std::dynamic_pointer_cast<Affine>(l)) {
         reads = writes = {af->data_mat.get()};
     } else if (auto ad = std::dynamic_pointer_cast<Add>(l)) {
@@ -283,8 +283,9 @@ static bool contains(const std::vector<const Mat *> &v, const Mat *m) {
 //     one pass of the float convolution.
 //  3. When the blob such a fused BinConv completes is the input of a later direct BinConv, the pass also writes that
 //     layer's packed input and the later layer skips its pack_mat.
-//  4. AvePool 2x2 stride 2 -> 1x1 FloatConv (the shortcut branch of a down-sampling block) becomes one launch that
-//     still writes the pooled blob.
+//  4. AvePool 2x2 stride 2 -> 1x1 FloatConv (the shortcut branch of a down-sampling block), the convolution being
+//     the only reader of the pooled blob, becomes one launch that does not write that blob: it leaves the net
+//     (get_blob says why).  With eight pooled pixels or fewer the blob stays and is written.
 //  5. FloatConv (-> Affine -> Relu) -> MaxPool 3x3 stride 2 pad 1, the pool being the only reader of the convolution's
 //     blob (the stem), becomes one pass that never writes that blob when the library says the pass pays for these
 //     shapes; the blob leaves the net (get_blob says why) and its memory, four times the pooled blob's, is freed.
@@ -423,6 +424,21 @@ void Net::fuse_binconv_epilogues() {
             continue;
         fc->fused_pool_input = pool->input_mat;
         fc->fused_pool_global = global;
+        // Nobody but this convolution reads the pooled blob, so the 2x2 form does not write it: the blob leaves the
+        // net (get_blob says why) and a Mat without memory keeps its shape for the layer.  Eight pooled pixels or
+        // fewer run as the two launches and keep the blob.
+        const Mat &pooled = *pool->output_mat;
+        if (!global && (long long)pooled.n * pooled.h * pooled.w > 8) {
+            for (auto it = mat_map_.begin(); it != mat_map_.end();) {
+                if (it->second == pool->output_mat) {
+                    elided_[it->first] = "the AvePool runs inside the convolution that reads it";
+                    it = mat_map_.erase(it);
+                } else {
+                    ++it;
+                }
+            }
+            fc->input_mat = std::make_shared<Mat>(pooled.n, pooled.h, pooled.w, pooled.c, nullptr, DataType::Float);
+        }
         layers.erase(layers.begin() + i);
         --i;
     }

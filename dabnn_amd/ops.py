@@ -268,8 +268,9 @@ def fconv_affine_relu(x, weight, bias, a, b, relu, kh, kw, pad_h, pad_w, stride_
     return out
 
 
-def ave_pool2_fconv1x1(x, weight, bias, a, b, relu):
-    """AvePool 2x2 stride 2 + 1x1 FpConv2D (+ Affine + Relu) in one launch; returns (pooled, out)."""
+def ave_pool2_fconv1x1(x, weight, bias, a, b, relu, want_pooled=True):
+    """AvePool 2x2 stride 2 + 1x1 FpConv2D (+ Affine + Relu) in one launch; returns (pooled, out), or (None, out)
+    without writing the pooled tensor when want_pooled is false."""
     _need(x, torch.float32, "x")
     _need(weight, torch.float32, "weight")
     n, h, w, c = x.shape
@@ -284,10 +285,10 @@ def ave_pool2_fconv1x1(x, weight, bias, a, b, relu):
             raise capi.DabError(capi.DAB_EINVAL, "ave_pool2_fconv1x1: %s does not match the channel count" % name)
         return _ptr(t)
     oh, ow = out_dim(h, 0, 2, 2), out_dim(w, 0, 2, 2)
-    pooled = _empty((n, max(oh, 0), max(ow, 0), c), torch.float32, x.device)
+    pooled = _empty((n, max(oh, 0), max(ow, 0), c), torch.float32, x.device) if want_pooled else None
     out = _empty((n, max(oh, 0), max(ow, 0), cout), torch.float32, x.device)
     check(lib.dab_ave_pool2_fconv1x1(_ptr(x), n, h, w, c, _ptr(weight), opt(bias, "bias"), opt(a, "a"), opt(b, "b"),
-                                     int(bool(relu)), cout, _ptr(pooled), _ptr(out), _stream()))
+                                     int(bool(relu)), cout, _ptr(pooled) if want_pooled else None, _ptr(out), _stream()))
     return pooled, out
 
 

@@ -220,6 +220,8 @@ DAB_API int dab_fconv_affine_relu(const float *x, int n, int h, int w, int c, co
  * (dabnn/fconv.h:14-76) and the optional Affine and Relu of dab_fconv_affine_relu, in one launch: the shortcut branch
  * of a down-sampling block.  pooled [n][(h-2)/2+1][(w-2)/2+1][c] receives the pooled tensor exactly as dab_ave_pool
  * writes it, out the convolution of it exactly as dab_fconv_affine_relu computes it from that tensor.
+ * pooled may be NULL when nobody reads the pooled tensor (it is then not written; out is the same), except for
+ * eight pooled pixels or fewer with cout >= 64, which run as the two launches and need the buffer (DAB_EINVAL).
  * wgt is [cout][1][1][c].  c must be a multiple of 4 and x, wgt, pooled 16-byte aligned (DAB_EUNSUPPORTED otherwise).
  */
 DAB_API int dab_ave_pool2_fconv1x1(const float *x, int n, int h, int w, int c, const float *wgt, const float *bias,

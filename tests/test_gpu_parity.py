@@ -721,6 +721,64 @@ def test_ave_pool2_fconv1x1_equals_the_two_layers(dab, n, h, w, c, cout, affine)
 
 
 @pytest.mark.parametrize("n,h,w,c,cout,bias,affine,relu", [
+    (8, 56, 56, 64, 128, False, True, False),    # the first shortcut branch of Bi-Real-18, whole tiles
+    (9, 30, 27, 64, 200, True, True, True),      # odd sizes: a ragged last pixel tile, a ragged second column tile
+    (11, 28, 28, 64, 72, True, False, True),     # one column tile, mostly empty
+    (2, 112, 112, 64, 384, False, False, False),  # three column tiles
+    (3, 28, 28, 128, 256, True, True, False)])   # 128 channels: the tile kernel, without the pooled tensor too
+def test_ave_pool2_fconv1x1_with_the_pooled_tile_in_lds(dab, n, h, w, c, cout, bias, affine, relu):
+    """64 input channels and enough pixels: a block pools its pixels once into LDS and walks the column tiles over
+    them.  Same bits as the two layers, with infinities, NaNs, signed zeros and denormals in the input, with every
+    epilogue, and the same convolution when the pooled tensor is not asked for."""
+    r = rng(47)
+    x = r.standard_normal((n, h, w, c)).astype(np.float32)
+    x.flat[::7] = 0.0
+    x.flat[3::11] = -0.0
+    x.flat[1::17] = np.float32(1e-45)
+    x.flat[2::19] = -np.float32(1e-45)
+    x.flat[::9973] = np.nan
+    x.flat[5::10007] = np.inf
+    x.flat[7::10009] = -np.inf
+
+    def same_bits(got, want):
+        got, want = got.cpu().numpy(), want.cpu().numpy()
+        np.testing.assert_array_equal(np.isnan(got), np.isnan(want))
+        np.testing.assert_array_equal(np.where(np.isnan(got), 0, got.view(np.uint32)), np.where(np.isnan(want), 0, want.view(np.uint32)))
+
+    wgt = (r.standard_normal((cout, 1, 1, c)) / np.sqrt(c)).astype(np.float32)
+    bv = r.standard_normal(cout).astype(np.float32)
+    a, b = r.standard_normal(cout).astype(np.float32), r.standard_normal(cout).astype(np.float32)
+    args = (dev_f(wgt), dev_f(bv) if bias else None, dev_f(a) if affine else None, dev_f(b) if affine else None, relu)
+    pooled, out = dab.ave_pool2_fconv1x1(dev_f(x), *args)
+    want_pooled = dab.ave_pool(dev_f(x), 2, 2, 0, 0, 2, 2)
+    want_out = dab.fconv_affine_relu(want_pooled, *args, 1, 1, 0, 0, 1, 1)
+    same_bits(pooled, want_pooled)
+    same_bits(out, want_out)
+    assert np.isfinite(want_out.cpu().numpy()).mean() > 0.3
+    none, out2 = dab.ave_pool2_fconv1x1(dev_f(x), *args, want_pooled=False)
+    assert none is None
+    same_bits(out2, want_out)
+    # against the CPU layers on finite data (sums of other orders: the tolerance of the float layers)
+    xf = r.standard_normal((2, h, w, c)).astype(np.float32)
+    _, got = dab.ave_pool2_fconv1x1(dev_f(xf), *args)
+    for i in range(2):
+        want = orc.fconv(orc.ave_pool(xf[i], 2, 2, 0, 0, 2, 2), wgt, bv if bias else None, 1, 1, 0, 0, 1, 1)
+        if affine:
+            want = orc.affine_inplace(want, a, b)
+        if relu:
+            want = orc.relu_inplace(want)
+        np.testing.assert_allclose(got[i].cpu().numpy(), want, rtol=1e-4, atol=1e-4 * np.abs(want).max())
+
+
+def test_ave_pool2_fconv1x1_needs_the_pooled_buffer_for_a_handful_of_pixels(dab):
+    x = torch.zeros((1, 4, 4, 64), device="cuda")
+    w = torch.zeros((64, 1, 1, 64), device="cuda")
+    with pytest.raises(RuntimeError):
+        dab.ave_pool2_fconv1x1(x, w, None, None, None, False, want_pooled=False)
+    dab.ave_pool2_fconv1x1(x, w, None, None, None, False)
+
+
+@pytest.mark.parametrize("n,h,w,c,cout,bias,affine,relu", [
     (1, 7, 7, 512, 1000, True, False, False),   # the end of Bi-Real-18 at batch 1
     (8, 7, 7, 512, 1000, False, False, False),  # the most images it takes
     (3, 8, 8, 1024, 64, True, True, True),      # the deepest and the largest window it takes, the fewest channels
