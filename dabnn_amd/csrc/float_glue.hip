@@ -35,7 +35,8 @@ namespace dab {
 // consecutive channels when the channel count is a multiple of 4.  POOL (1x1
 // convolutions with CV = 4) averages 2x2 windows of the input on the way in --
 // an AvePool 2x2 stride 2 followed by the convolution, the shortcut branch of a
-// down-sampling block, in one launch; the pooled tensor is still written.
+// down-sampling block, in one launch; the pooled tensor is written too unless
+// p.pooled is null.
 struct FconvArgs {
     const float *x;
     const float *w;

@@ -48,7 +48,8 @@ class BNN_API FloatConv : public Layer {
     MatP fused_a, fused_b;
     bool fused_relu = false;
     // Set by Net::prepare for a 1x1 convolution that reads the output of an AvePool 2x2 stride 2: the pool's input.
-    // The layer then pools it itself, writes the pooled blob (input_mat) as a side product and convolves it.
+    // The layer then pools it itself and convolves the result; the pooled blob (input_mat) is written as a side product
+    // when it has device memory, and is a shape without memory when the net dropped the blob.
     MatP fused_pool_input;
     // The same for a global AvePool (one window over the whole image) at small batch: fused_pool_input is its input.
     bool fused_pool_global = false;
