@@ -51,15 +51,29 @@ Mat::~Mat() {
     if (dev && !external_memory) (void)hipFree(dev);
 }
 
+// Copies between host and device go over one stream of their own that does not synchronise with the null stream, and
+// wait for it.  A plain hipMemcpy works on the null stream, and a null-stream operation issued by one thread while
+// another thread's Net captures its HIP graph fails and invalidates that capture.
+static hipStream_t copy_stream() {
+    static hipStream_t s = [] {
+        hipStream_t created = nullptr;
+        hip_check(hipStreamCreateWithFlags(&created, hipStreamNonBlocking), "hipStreamCreate");
+        return created;
+    }();
+    return s;
+}
+
 void Mat::upload(const void *host, size_t nbytes) {
     if (nbytes > bytes()) throw std::runtime_error("Mat::upload: source larger than the tensor");
-    hip_check(hipMemcpy(dev, host, nbytes, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    hip_check(hipMemcpyAsync(dev, host, nbytes, hipMemcpyHostToDevice, copy_stream()), "hipMemcpyAsync H2D");
+    hip_check(hipStreamSynchronize(copy_stream()), "hipStreamSynchronize");
     host_valid_ = false;
 }
 
 void Mat::download(void *host, size_t nbytes) const {
     if (nbytes > bytes()) throw std::runtime_error("Mat::download: destination larger than the tensor");
-    hip_check(hipMemcpy(host, dev, nbytes, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    hip_check(hipMemcpyAsync(host, dev, nbytes, hipMemcpyDeviceToHost, copy_stream()), "hipMemcpyAsync D2H");
+    hip_check(hipStreamSynchronize(copy_stream()), "hipStreamSynchronize");
 }
 
 std::vector<float> Mat::to_host_float() const {
@@ -82,8 +96,7 @@ void Mat::sync_to_host() const {
         host_.resize(bytes());
         data = host_.empty() ? nullptr : host_.data();
     }
-    // hipMemcpy waits for work queued on other streams of this device to have finished with the memory it reads
-    // only if that work was submitted to the null stream; a Net synchronises its own stream at the end of run()
+    // the copy does not wait for work queued on other streams; a Net synchronises its own stream at the end of run()
     if (!host_.empty()) download(host_.data(), host_.size());
     host_valid_ = true;
 }

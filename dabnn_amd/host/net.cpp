@@ -5,6 +5,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <fstream>
+#include <mutex>
 #include <sstream>
 #include <stdexcept>
 
@@ -45,6 +46,14 @@ void Layer::forward() {
 }
 
 // ---------------------------------------------------------------- Net
+// Nets of one process may run on host threads of their own.  A net captures its HIP graph on its third run; device
+// allocations and frees of other threads (a net being read or destroyed) and a second capture stay out of that
+// window.  Kernel launches and copies of other nets do not take the lock.
+static std::mutex &capture_mutex() {
+    static std::mutex m;
+    return m;
+}
+
 Net::Net() {
     hipStream_t s;
     hip_check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
@@ -52,6 +61,7 @@ Net::Net() {
 }
 
 Net::~Net() {
+    std::lock_guard<std::mutex> lock(capture_mutex());
     if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
     layers.clear();
     mat_map_.clear();
@@ -116,6 +126,7 @@ std::shared_ptr<Mat> Net::blob(const std::string &name) {
 }
 
 void Net::prepare(const void *buf, size_t len) {
+    std::lock_guard<std::mutex> lock(capture_mutex());
     BNN_ASSERT(!prepared_, "a Net can be read once");
     BNN_ASSERT(!(strict && !run_fconv), "fconv must be run in strict mode");
     // parse (bounds-checked) and check the whole model on the host before anything is allocated on the device
@@ -501,6 +512,7 @@ void Net::run_device(const void *device_input) {
         hip_check(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec_), s), "hipGraphLaunch");
     } else if (runs_ >= 2) {
         // capture the kernels of one forward pass; nothing in the layers allocates, synchronises or memsets
+        std::lock_guard<std::mutex> lock(capture_mutex());
         hipGraph_t graph = nullptr;
         hip_check(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
         try {
