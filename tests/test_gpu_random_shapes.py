@@ -155,3 +155,45 @@ def test_fconv_over_32_channels_on_random_shapes(dab):
         y = y.permute(0, 2, 3, 1)
         assert got.shape == y.shape, case
         assert (got.double() - y).abs().max().item() <= 4e-6 * y.abs().max().item(), case
+
+
+@pytest.mark.parametrize("seed", range(2))
+def test_pooled_shortcut_convolution_on_random_shapes(dab, seed):
+    """AvePool 2x2 stride 2 + 1x1 FpConv2D (+ bias, Affine, Relu) in one launch (dabnn/layers/AvePool.cpp:84-123,
+    dabnn/fconv.h:14-76): over 64 channels with enough pixels the kernel that keeps a block's pooled pixels in LDS,
+    otherwise the tile kernel with the pooling loader.  Pooled tensor and convolution bit for bit those of the two
+    separate launches, the same convolution without the pooled tensor, and both within the float tolerance of the
+    CPU layers."""
+    r = np.random.default_rng(500 + seed)
+    for case_no in range(12):
+        if case_no < 7:  # 64 channels and thousands of pooled pixels: the pooled tile in LDS
+            c, n, h, w = 64, int(r.integers(6, 25)), int(r.integers(30, 60)), int(r.integers(30, 60))
+            cout = int(r.choice([65, 72, 128, 130, 200, 256, 384]))
+        else:
+            c = int(r.choice([64, 64, 128, 32, 8]))
+            n, h, w = int(r.integers(1, 12)), int(r.integers(2, 60)), int(r.integers(2, 60))
+            cout = int(r.choice([65, 72, 128, 130, 200, 256, 384, 17]))
+        flags = [bool(r.random() < 0.5) for _ in range(3)]
+        case = "n %d h %d w %d c %d cout %d bias %d affine %d relu %d" % (n, h, w, c, cout, *flags)
+        x = r.standard_normal((n, h, w, c)).astype(np.float32)
+        wgt = (r.standard_normal((cout, 1, 1, c)) / np.sqrt(c)).astype(np.float32)
+        bias, a, b = (r.standard_normal(cout).astype(np.float32) for _ in range(3))
+        args = (dev_f(wgt), dev_f(bias) if flags[0] else None, dev_f(a) if flags[1] else None,
+                dev_f(b) if flags[1] else None, flags[2])
+        pooled, out = dab.ave_pool2_fconv1x1(dev_f(x), *args)
+        want_pooled = dab.ave_pool(dev_f(x), 2, 2, 0, 0, 2, 2)
+        want_out = dab.fconv_affine_relu(want_pooled, *args, 1, 1, 0, 0, 1, 1)
+        np.testing.assert_array_equal(pooled.cpu().numpy(), want_pooled.cpu().numpy(), err_msg=case)
+        np.testing.assert_array_equal(out.cpu().numpy(), want_out.cpu().numpy(), err_msg=case)
+        if n * (h // 2) * (w // 2) > 8 or cout < 64:
+            _, out2 = dab.ave_pool2_fconv1x1(dev_f(x), *args, want_pooled=False)
+            np.testing.assert_array_equal(out2.cpu().numpy(), want_out.cpu().numpy(), err_msg=case)
+        for i in range(min(n, 2)):
+            cpu_pooled = orc.ave_pool(x[i], 2, 2, 0, 0, 2, 2)
+            np.testing.assert_array_equal(pooled[i].cpu().numpy(), cpu_pooled, err_msg=case)
+            want = orc.fconv(cpu_pooled, wgt, bias if flags[0] else None, 1, 1, 0, 0, 1, 1)
+            if flags[1]:
+                want = orc.affine_inplace(want, a, b)
+            if flags[2]:
+                want = orc.relu_inplace(want)
+            np.testing.assert_allclose(out[i].cpu().numpy(), want, rtol=RTOL, atol=RTOL * np.abs(want).max(), err_msg=case)
