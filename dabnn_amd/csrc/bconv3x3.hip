@@ -697,7 +697,7 @@ __global__ __launch_bounds__(256, 6) void bconv3x3_tile64_kernel(const BconvArgs
                 const bool ok = tile * 64 + pixel < p.total;
                 if (ok) {
                     typedef float f32x4 __attribute__((ext_vector_type(4)));
-                    DAB_EPI_STORE((f32x4{r.x, r.y, r.z, r.w}), reinterpret_cast<f32x4 *>(p.out + out_off + j * step));
+                    __builtin_nontemporal_store(f32x4{r.x, r.y, r.z, r.w}, reinterpret_cast<f32x4 *>(p.out + out_off + j * step));
                 }
                 if constexpr (MODE == kModeAffineAddSign) {
                     // the 16 lanes of a pixel are one row of lanes

@@ -297,16 +297,6 @@ struct EpiAffineAddSign : EpiAffineAdd {
 // every piece leaves the L2 once, as it arrives: the counter reads the output size, a launch ends 0.3-1.6 us earlier
 // at batch 64 and the next one starts on an L2 with nothing left to write.  Small outputs stay in the L2s either
 // way and are 0.2-0.6 us faster with the streaming stores, so the launcher asks for this above a size.
-#ifndef DAB_EPI_ST
-#define DAB_EPI_ST 0
-#endif
-#if DAB_EPI_ST == 0
-#define DAB_EPI_STORE(v, d) __builtin_nontemporal_store(v, d)
-#elif DAB_EPI_ST == 1
-#define DAB_EPI_STORE(v, d) (*(d) = (v))
-#else
-#define DAB_EPI_STORE(v, d) store_through(d, v)
-#endif
 template <int WCH, int G, bool SC, bool THROUGH, class Epi>
 __device__ __forceinline__ void stage_flush_window(const unsigned char *stage, int lane, float *__restrict__ out, int ld,
                                                    int tile, int cbase, Epi &epi) {
@@ -341,7 +331,7 @@ __device__ __forceinline__ void stage_flush_window(const unsigned char *stage, i
             else
                 // streaming store: the output is not read again by this kernel, and lines that leave the L2 early
                 // do not have to be written back when the kernel ends
-                DAB_EPI_STORE(rv, dst);
+                __builtin_nontemporal_store(rv, dst);
             if constexpr (Epi::kEmit) {
                 // the NP lanes of a pixel hold its window's sign bits, four each: gather them in the first lane
                 uint32_t w = sign_nibble(r) << (4 * part);
@@ -375,7 +365,7 @@ __device__ __forceinline__ void stage_flush(const unsigned char *stage, int lane
     // how the stores go through the L2 is the launch's choice (EpiStore), one way for all of them
     bool through = false;
     if constexpr (Epi::kPolicy) through = epi.through != 0;
-    const bool parts_through = through || (DAB_EPI_ST == 3 && !Epi::kPolicy);
+    const bool parts_through = through;
     if (np == NP && (tile + 1) * 64 <= total) {
         if (has_sc)
             stage_flush_window<WCH, GG, Epi::kShortcut, false>(stage, lane, out, ld, tile, cbase, epi);
