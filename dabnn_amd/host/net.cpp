@@ -63,6 +63,7 @@ Net::Net() {
 Net::~Net() {
     std::lock_guard<std::mutex> lock(capture_mutex());
     if (graph_exec_) (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
+    if (input_own_dev_ && mat_map_.count(input_name_)) mat_map_[input_name_]->dev = input_own_dev_;  // freed by its Mat
     layers.clear();
     mat_map_.clear();
     if (stream_) (void)hipStreamDestroy(static_cast<hipStream_t>(stream_));
@@ -145,6 +146,7 @@ void Net::prepare(const void *buf, size_t len) {
         const InputDesc &in = model.inputs[0];
         input_name_ = in.name;
         add_mat(input_name_, std::make_shared<Mat>(batch_, in.shape[1], in.shape[2], in.shape[3], DataType::Float, input_name_));
+        input_own_dev_ = mat_map_[input_name_]->dev;
     }
 
     // initializers (dabnn/net.cpp:72-138), uploaded to the device
@@ -238,6 +240,8 @@ void Net::prepare(const void *buf, size_t len) {
         }
     }
     if (optimize) fuse_binconv_epilogues();
+    // an in-place layer on the input blob would write into a caller's buffer that is read in place
+    copy_input_ = layers_write_input();
     hip_check(hipStreamSynchronize(static_cast<hipStream_t>(stream_)), "hipStreamSynchronize");
     prepared_ = true;
 }
@@ -277,6 +281,17 @@ static void layer_io(const std::shared_ptr<Layer> &l, std::vector<const Mat *> &
     } else if (auto sh = std::dynamic_pointer_cast<Shuffle>(l)) {
         reads = writes = {sh->data_mat.get()};
     }
+}
+
+bool Net::layers_write_input() {
+    std::vector<const Mat *> rd, wr;
+    const Mat *in = blob(input_name_).get();
+    for (const auto &l : layers) {
+        layer_io(l, rd, wr);
+        for (const Mat *m : wr)
+            if (m == in) return true;
+    }
+    return false;
 }
 
 static bool contains(const std::vector<const Mat *> &v, const Mat *m) {
@@ -492,20 +507,46 @@ void Net::fuse_binconv_epilogues() {
 void Net::run(const void *host_input) {
     BNN_ASSERT(prepared_, "run before read");
     BNN_ASSERT(host_input != nullptr, "run: null input");
+    bind_input(nullptr);
     auto in = blob(input_name_);
     hip_check(hipMemcpyAsync(in->dev, host_input, in->bytes(), hipMemcpyHostToDevice, static_cast<hipStream_t>(stream_)),
               "hipMemcpyAsync");
-    run_device(nullptr);
+    launch_layers();
 }
 
 void Net::run_device(const void *device_input) {
     BNN_ASSERT(prepared_, "run before read");
+    bind_input(device_input);
+    launch_layers();
+}
+
+// Points the input blob at the memory this run reads: the caller's device buffer in place, or the blob's own
+// allocation (host inputs, unaligned buffers, callers whose buffers keep changing), filled here from device_input.
+void Net::bind_input(const void *device_input) {
+    auto in = blob(input_name_);
+    const bool in_place = device_input != nullptr && !copy_input_ && reinterpret_cast<uintptr_t>(device_input) % 256 == 0;
+    void *want = in_place ? const_cast<void *>(device_input) : input_own_dev_;
+    if (graph_exec_ && graph_input_ != want) {
+        // the graph's kernels hold the address they were captured with
+        if (in_place && ++input_rebinds_ >= 3) {
+            copy_input_ = true;
+            want = input_own_dev_;
+        }
+        if (graph_input_ != want) {
+            std::lock_guard<std::mutex> lock(capture_mutex());
+            (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec_));
+            graph_exec_ = nullptr;
+        }
+    }
+    in->dev = want;
+    if (device_input != nullptr && want == input_own_dev_)
+        hip_check(hipMemcpyAsync(in->dev, device_input, in->bytes(), hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream_)),
+                  "hipMemcpyAsync");
+}
+
+void Net::launch_layers() {
     BNN_ASSERT(!(strict && !run_fconv), "fconv must be run in strict mode");
     hipStream_t s = static_cast<hipStream_t>(stream_);
-    if (device_input) {
-        auto in = blob(input_name_);
-        hip_check(hipMemcpyAsync(in->dev, device_input, in->bytes(), hipMemcpyDeviceToDevice, s), "hipMemcpyAsync");
-    }
     if (profile || !use_graph) {
         for (const auto &layer : layers) layer->forward();
     } else if (graph_exec_) {
@@ -527,6 +568,7 @@ void Net::run_device(const void *device_input) {
         hip_check(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate");
         (void)hipGraphDestroy(graph);
         graph_exec_ = exec;
+        graph_input_ = blob(input_name_)->dev;
         hip_check(hipGraphLaunch(exec, s), "hipGraphLaunch");
     } else {
         for (const auto &layer : layers) layer->forward();

@@ -6,7 +6,8 @@
 // All blobs live in device memory; run() takes a HOST pointer to
 // batch x H x W x C floats (NHWC) like the reference's run(void*), uploads it,
 // enqueues every layer on the net's stream and waits.  run_device() takes a
-// device pointer and skips the copy.
+// device pointer and reads the input in place (as the reference's run wraps
+// its host pointer without a copy).
 #pragma once
 
 #include <map>
@@ -31,6 +32,11 @@ class BNN_API Net : public std::enable_shared_from_this<Net> {
     void read_buf(const void *ptr);
     void read_buf(const void *ptr, size_t len);  // the same, with every offset of the model checked against len
     void run(const void *host_input);
+    // The layers read device_input where it lies, which must stay valid and unchanged until the call returns (256-byte
+    // aligned, as hipMalloc gives it; anything else is copied into the net's own input blob).  The HIP graph holds
+    // the address it was captured with: the same buffer run after run replays it, another buffer makes the net
+    // capture again, and from the third such change on the net copies every input into its own blob instead.
+    // nullptr: the input blob already holds the input.
     void run_device(const void *device_input);
     // The blob with its host mirror up to date (dabnn/net.cpp:288-290): `data`, operator[] ... read what the last
     // run left on the device.
@@ -77,6 +83,13 @@ class BNN_API Net : public std::enable_shared_from_this<Net> {
     bool prepared_ = false;
     int runs_ = 0;
     void *graph_exec_ = nullptr;
+    void *input_own_dev_ = nullptr;       // the input blob's own allocation
+    const void *graph_input_ = nullptr;   // the input address the graph's kernels hold
+    int input_rebinds_ = 0;               // captures thrown away because the caller's buffer changed
+    bool copy_input_ = false;             // the caller's buffers keep changing: copy into the own blob
+    void bind_input(const void *device_input);
+    bool layers_write_input();
+    void launch_layers();
 };
 
 }  // namespace bnn

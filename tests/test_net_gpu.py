@@ -600,3 +600,75 @@ def test_nets_on_threads_of_their_own_do_not_disturb_each_other(mods):
         for k, one_round in enumerate(got[i]):
             for j, (g, w) in enumerate(zip(one_round, alone[i])):
                 np.testing.assert_array_equal(g, w, err_msg="thread %d round %d run %d" % (i, k, j))
+
+
+def test_run_device_reads_the_callers_buffer_in_place(mods):
+    """A device input is read where it lies (the reference's run wraps its pointer without a copy): the same buffer
+    run after run replays the captured graph and sees new contents, another buffer makes the net capture again, from
+    the third change on the net copies into its own blob, and an unaligned buffer is copied from the start.  Every
+    run gives the logits of the same input passed from the host."""
+    import torch
+    df, models, net = mods
+    layers, inits, inputs = models.small_bnn(6, hw=16, width=64)
+    buf = df.write_model(layers, inits, inputs)
+    r = np.random.default_rng(17)
+    batch = 3
+    xs = [r.standard_normal((batch, 16, 16, 3)).astype(np.float32) for _ in range(12)]
+    ref = net.Net(batch=batch).read_buf(buf)
+    ref.set_use_graph(False)
+    want = [ref.run(x).get_blob("logits").copy() for x in xs]
+    ref.close()
+
+    n = net.Net(batch=batch).read_buf(buf)
+    a = torch.empty((batch, 16, 16, 3), device="cuda")
+    keep = a.clone()
+    for i in range(5):  # one buffer, new contents every run: two eager runs, the capture, two replays
+        a.copy_(torch.from_numpy(xs[i]))
+        keep.copy_(a)
+        np.testing.assert_array_equal(n.run(a).get_blob("logits"), want[i], err_msg="run %d" % i)
+        assert torch.equal(a, keep), "the net wrote into the caller's buffer"
+        np.testing.assert_array_equal(n.get_blob(n.input_name), xs[i])
+    others = [torch.from_numpy(xs[i]).cuda() for i in range(5, 10)]  # a new buffer every run
+    for i, t in zip(range(5, 10), others):
+        np.testing.assert_array_equal(n.run(t).get_blob("logits"), want[i], err_msg="run %d" % i)
+        np.testing.assert_array_equal(n.get_blob(n.input_name), xs[i])
+    np.testing.assert_array_equal(n.run(xs[10]).get_blob("logits"), want[10])  # a host input in between
+    flat = torch.empty(batch * 16 * 16 * 3 + 8, device="cuda")
+    odd = flat[1:1 + batch * 16 * 16 * 3].view(batch, 16, 16, 3)  # four bytes off the allocation's alignment
+    assert odd.data_ptr() % 256 != 0 and odd.is_contiguous()
+    odd.copy_(torch.from_numpy(xs[11]))
+    np.testing.assert_array_equal(n.run(odd).get_blob("logits"), want[11])
+    np.testing.assert_array_equal(n.run(a).get_blob("logits"), want[4])
+    n.close()
+
+    # a fresh net, an unaligned buffer from the first run on and through the capture
+    m = net.Net(batch=batch).read_buf(buf)
+    for i in range(4):
+        odd.copy_(torch.from_numpy(xs[i]))
+        np.testing.assert_array_equal(m.run(odd).get_blob("logits"), want[i], err_msg="run %d" % i)
+    m.close()
+
+
+def test_run_device_copies_when_a_layer_rewrites_the_input_blob(mods):
+    """An in-place layer on the input blob (an Affine that normalises the image) must not write into the caller's
+    device buffer: such a net copies its input."""
+    import torch
+    df, models, net = mods
+    r = np.random.default_rng(19)
+    a, b = r.standard_normal(4).astype(np.float32), r.standard_normal(4).astype(np.float32)
+    w = (r.standard_normal((8, 3, 3, 4)) / 6).astype(np.float32)
+    inits = [{"name": "a", "shape": [4], "data": a, "align_hwc_to_128": False},
+             {"name": "b", "shape": [4], "data": b, "align_hwc_to_128": False},
+             {"name": "w", "shape": [8, 3, 3, 4], "data": w, "align_hwc_to_128": False}]
+    layers = [{"type": "Affine", "name": "norm", "input": "data", "a": "a", "b": "b", "output": "data_n"},
+              {"type": "FpConv2D", "name": "conv", "input": "data_n", "weight": "w", "output": "conv_out", "pads": [1] * 4,
+               "strides": [1, 1], "dilations": [1, 1]}]
+    n = net.Net(batch=2).read_buf(df.write_model(layers, inits, [("data", [1, 9, 9, 4])]))
+    x = r.standard_normal((2, 9, 9, 4)).astype(np.float32)
+    t = torch.from_numpy(x).cuda()
+    for _ in range(4):
+        got = n.run(t).get_blob("conv_out")
+        assert torch.equal(t.cpu(), torch.from_numpy(x)), "the net wrote into the caller's buffer"
+        for i in range(2):
+            close(got[i], orc.fconv(orc.affine_inplace(x[i].copy(), a, b), w, None, 3, 3, 1, 1, 1, 1))
+    n.close()
