@@ -66,7 +66,13 @@ DABNET_API int dabnet_check_model(const void *buf, size_t len, int run_fconv);
 
 /* Net::run (dabnn/net.cpp:272-286): host_input holds batch x H x W x C floats (NHWC). Blocks until done. */
 DABNET_API int dabnet_run(dabnet_t *net, const float *host_input);
-/* Same with the input already in device memory. */
+/*
+ * Same with the input already in device memory.  The layers read device_input where it lies (the reference's run wraps
+ * its pointer without a copy), so it must stay valid and unchanged until the call returns; the net does not write to
+ * it.  It is copied into the net's own input blob instead when it is not 256-byte aligned, when a layer rewrites the
+ * input blob in place, or from the third time on that the address differs from the one the net's HIP graph was
+ * captured with (a change of address costs a new capture).  NULL: the input blob already holds the input.
+ */
 DABNET_API int dabnet_run_device(dabnet_t *net, const float *device_input);
 
 /* Name of the model's input blob (its shape through dabnet_blob_info). */
