@@ -98,7 +98,8 @@ class Net:
         return self
 
     def run(self, x):
-        """x: host array of batch x H x W x C float32 (NHWC), or a CUDA torch tensor of that shape."""
+        """x: host array of batch x H x W x C float32 (NHWC), or a CUDA torch tensor of that shape, which the layers
+        read in place (reuse one tensor run after run: the net's HIP graph holds its address)."""
         if hasattr(x, "is_cuda") and x.is_cuda:
             import torch
             assert x.dtype == torch.float32 and x.is_contiguous()
