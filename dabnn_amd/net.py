@@ -73,6 +73,7 @@ class Net:
         if not self._h:
             raise RuntimeError(hostlib.dabnet_last_error().decode())
         self.batch = batch
+        self._input_bytes = None  # of the input blob, asked for once
         _check(hostlib.dabnet_set_batch(self._h, batch))
         _check(hostlib.dabnet_set_flags(self._h, int(optimize), int(run_fconv), int(strict)))
 
@@ -103,7 +104,9 @@ class Net:
         if hasattr(x, "is_cuda") and x.is_cuda:
             import torch
             assert x.dtype == torch.float32 and x.is_contiguous()
-            if x.numel() * 4 != self.blob_info(self.input_name)[2]:
+            if self._input_bytes is None:
+                self._input_bytes = self.blob_info(self.input_name)[2]
+            if x.numel() * 4 != self._input_bytes:
                 raise ValueError("input tensor does not match the model's input size")
             torch.cuda.current_stream().synchronize()
             _check(hostlib.dabnet_run_device(self._h, ctypes.c_void_p(x.data_ptr())))
