@@ -539,7 +539,7 @@ void Net::bind_input(const void *device_input) {
         }
     }
     in->dev = want;
-    if (device_input != nullptr && want == input_own_dev_)
+    if (device_input != nullptr && want == input_own_dev_ && device_input != input_own_dev_)
         hip_check(hipMemcpyAsync(in->dev, device_input, in->bytes(), hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream_)),
                   "hipMemcpyAsync");
 }
