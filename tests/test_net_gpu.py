@@ -558,50 +558,6 @@ def test_graph_replay_equals_eager(mods):
     graphed.close()
 
 
-def test_nets_on_threads_of_their_own_do_not_disturb_each_other(mods):
-    """Every Net has a stream of its own: nets that are read, run (eager runs, the capture of the HIP graph on the
-    third run, replays), read back and destroyed on two host threads at once give the logits each gives alone."""
-    import threading
-    df, models, net = mods
-    layers, inits, inputs = models.bireal18(21, stem=False)
-    buf = df.write_model(layers, inits, inputs)
-    r = np.random.default_rng(13)
-    batches = (3, 8)
-    xs = [[r.standard_normal((b, 224, 224, 3)).astype(np.float32) for _ in range(5)] for b in batches]
-    alone = []
-    for b, inputs_ in zip(batches, xs):
-        ref = net.Net(batch=b).read_buf(buf)
-        ref.set_use_graph(False)
-        alone.append([ref.run(x).get_blob("logits").copy() for x in inputs_])
-        ref.close()
-    rounds = 4
-    got = [[], []]
-    errors = []
-    start = threading.Barrier(2)
-
-    def work(i):
-        try:
-            start.wait()
-            for _ in range(rounds):
-                n = net.Net(batch=batches[i]).read_buf(buf)
-                got[i].append([n.run(x).get_blob("logits").copy() for x in xs[i]])
-                n.close()
-        except Exception as e:  # noqa: BLE001 - reported by the assertion below
-            errors.append("thread %d: %r" % (i, e))
-
-    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
-    for t in threads:
-        t.start()
-    for t in threads:
-        t.join()
-    assert not errors, errors
-    for i in range(2):
-        assert len(got[i]) == rounds
-        for k, one_round in enumerate(got[i]):
-            for j, (g, w) in enumerate(zip(one_round, alone[i])):
-                np.testing.assert_array_equal(g, w, err_msg="thread %d round %d run %d" % (i, k, j))
-
-
 def test_run_device_reads_the_callers_buffer_in_place(mods):
     """A device input is read where it lies (the reference's run wraps its pointer without a copy): the same buffer
     run after run replays the captured graph and sees new contents, another buffer makes the net capture again, from
@@ -672,3 +628,47 @@ def test_run_device_copies_when_a_layer_rewrites_the_input_blob(mods):
         for i in range(2):
             close(got[i], orc.fconv(orc.affine_inplace(x[i].copy(), a, b), w, None, 3, 3, 1, 1, 1, 1))
     n.close()
+
+
+def test_nets_on_threads_of_their_own_do_not_disturb_each_other(mods):
+    """Every Net has a stream of its own: nets that are read, run (eager runs, the capture of the HIP graph on the
+    third run, replays), read back and destroyed on two host threads at once give the logits each gives alone."""
+    import threading
+    df, models, net = mods
+    layers, inits, inputs = models.bireal18(21, stem=False)
+    buf = df.write_model(layers, inits, inputs)
+    r = np.random.default_rng(13)
+    batches = (3, 8)
+    xs = [[r.standard_normal((b, 224, 224, 3)).astype(np.float32) for _ in range(5)] for b in batches]
+    alone = []
+    for b, inputs_ in zip(batches, xs):
+        ref = net.Net(batch=b).read_buf(buf)
+        ref.set_use_graph(False)
+        alone.append([ref.run(x).get_blob("logits").copy() for x in inputs_])
+        ref.close()
+    rounds = 4
+    got = [[], []]
+    errors = []
+    start = threading.Barrier(2)
+
+    def work(i):
+        try:
+            start.wait()
+            for _ in range(rounds):
+                n = net.Net(batch=batches[i]).read_buf(buf)
+                got[i].append([n.run(x).get_blob("logits").copy() for x in xs[i]])
+                n.close()
+        except Exception as e:  # noqa: BLE001 - reported by the assertion below
+            errors.append("thread %d: %r" % (i, e))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i in range(2):
+        assert len(got[i]) == rounds
+        for k, one_round in enumerate(got[i]):
+            for j, (g, w) in enumerate(zip(one_round, alone[i])):
+                np.testing.assert_array_equal(g, w, err_msg="thread %d round %d run %d" % (i, k, j))
