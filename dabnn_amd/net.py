@@ -82,9 +82,9 @@ class Net:
         return cls(**kw)
 
     def close(self):
-        if self._h:
+        if self._h and hostlib is not None:  # at interpreter exit the module's globals may be gone already
             hostlib.dabnet_destroy(self._h)
-            self._h = None
+        self._h = None
 
     def __del__(self):
         self.close()
